@@ -1,11 +1,13 @@
 """One registry from an architecture's name (config.json `architectures[0]`, or `architecture`) to
 its typed configuration, and through `to_spec()` to its model.  A configuration
 class offers `from_dict(config_json) -> cfg`, `cfg.to_dict()`, `cfg.to_spec()
--> ModelSpec` and optionally `cfg.with_window(n)`."""
+-> ModelSpec` and optionally `cfg.with_window(n)` and `cfg.with_tensor_shapes(shape_of)` (a design that leaves
+sizes to the shapes of a folder's tensors: `config_from_folder` calls it with the folder's shapes)."""
 import json
 import os
 
 from .llama import ConfigError, LlamaConfig
+from .bovozen import BovozenConfig
 from .gedunex import GedunexConfig
 from .situlorn import SitulornConfig
 
@@ -41,9 +43,26 @@ def config_from_folder(path):
     if not os.path.exists(f):
         raise ConfigError("no config.json in %s" % path)                # convert.py:223-224
     with open(f) as fh:
-        return config_from_dict(json.load(fh))
+        cfg = config_from_dict(json.load(fh))
+    if hasattr(cfg, "with_tensor_shapes"):
+        cfg = cfg.with_tensor_shapes(_folder_shapes(path))
+    return cfg
 
 
-for _cls in (LlamaConfig, SitulornConfig, GedunexConfig):
+def _folder_shapes(path):
+    """name -> shape (or None) over the headers of a folder's *.safetensors files; no tensor is read."""
+    from ..weights.safetensors_io import SafetensorsError, SafetensorsFile
+    shapes = {}
+    for n in sorted(os.listdir(path)):
+        if n.endswith(".safetensors"):
+            try:
+                for key, entry in SafetensorsFile(os.path.join(path, n)).entries.items():
+                    shapes[key] = tuple(entry.shape)
+            except SafetensorsError:
+                pass                        # the loader reports a broken file with its own words
+    return shapes.get
+
+
+for _cls in (LlamaConfig, SitulornConfig, GedunexConfig, BovozenConfig):
     for _name in _cls.ARCHITECTURES:
         register_architecture(_name, _cls)

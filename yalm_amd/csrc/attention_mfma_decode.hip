@@ -54,7 +54,7 @@ __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_k
   for (int dt = 0; dt < DT; ++dt) o[dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
   if (L > 0) {
-    const int lo = window > 0 ? max(0, L - window) : 0;
+    const int lo = first_visible(L - 1, window, shape.block);
     const int first_page = lo / PAGE, last_page = (L - 1) / PAGE;
     const int total = last_page - first_page + 1;
     int per = (total + n_splits - 1) / n_splits;
@@ -64,7 +64,7 @@ __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_k
       // instead of every sequence cutting its own length into n_splits pieces of unequal cost.  Whatever the value
       // says, the sequence's own pages are all covered.
       const int Lm = max(step_max_len[0], 1);
-      const int total_m = (Lm - 1) / PAGE - (window > 0 ? max(0, Lm - window) / PAGE : 0) + 1;
+      const int total_m = (Lm - 1) / PAGE - first_visible(Lm - 1, window, shape.block) / PAGE + 1;
       per = max(per, (total_m + n_splits - 1) / n_splits);
     }
     const int p_begin = first_page + split * per;

@@ -105,7 +105,13 @@ __global__ __launch_bounds__(256 * KSPL, KSPL == 1 ? 2 : 1) void attn_prefill_mf
 
   const int blk_last = min(blk0 + NC * PAGE - 1, len - 1);
   const int kt_hi = blk_last / PAGE;
-  const int kt_lo = window > 0 ? max(0, blk0 - window + 1) / PAGE : 0;
+  const int block = shape.block;                  // a query sees its own block of positions only (0: no blocks)
+  const int kt_lo = first_visible(blk0, window, block) / PAGE;
+  int lo_q[NC];                                   // the first position each query sees
+#pragma unroll
+  for (int c = 0; c < NC; ++c) lo_q[c] = first_visible(pos_q[c], window, block);
+  const int wave_lo = first_visible(pos0, window, block);                       // the least of the wave's queries'
+  const int wave_lo_last = first_visible(pos0 + 16 * NC - 1, window, block);    // and the greatest
   const int wave_last = min(pos0 + 16 * NC - 1, len - 1);
   const size_t tile_elems = (size_t)n_kv_heads * PAGE * HD;
 
@@ -147,8 +153,7 @@ __global__ __launch_bounds__(256 * KSPL, KSPL == 1 ? 2 : 1) void attn_prefill_mf
     const bool next = kt + KSPL <= kt_hi;
     if (next) load_tile(kt + KSPL);
     const int base = kt * PAGE;
-    const bool visible = kt <= kt_hi && wave_live && base <= wave_last &&
-                         (window == 0 || base + PAGE - 1 > pos0 - window);
+    const bool visible = kt <= kt_hi && wave_live && base <= wave_last && base + PAGE - 1 >= wave_lo;
     if (visible) {
       const bf16* ks_l = smem + (cur * KSPL + half) * (KTILE + VTILE);
       const bf16* vs_l = ks_l + KTILE;
@@ -166,7 +171,7 @@ __global__ __launch_bounds__(256 * KSPL, KSPL == 1 ? 2 : 1) void attn_prefill_mf
           for (int c = 0; c < NC; ++c)
             sc[c][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qv[c][ks], sc[c][t], 0, 0, 0);
         }
-      const bool edge = base + PAGE - 1 > pos0 || (window > 0 && base < pos0 + 16 * NC - 1 - window + 1);
+      const bool edge = base + PAGE - 1 > pos0 || base < wave_lo_last;
       bf16x8 pb[NC][2];
       float corr[NC];
       // scores in the base-2 domain: p = 2^(s * log2(e) / sqrt(hd) - m)
@@ -193,7 +198,7 @@ __global__ __launch_bounds__(256 * KSPL, KSPL == 1 ? 2 : 1) void attn_prefill_mf
               }
               if (decltype(masked)::value) {
                 int kpos = base + 32 * (t >> 1) + 8 * qd + 4 * (t & 1) + r;
-                bool vis = kpos <= pos_q[c] && (window == 0 || pos_q[c] - kpos < window) && q_ok[c];
+                bool vis = kpos <= pos_q[c] && kpos >= lo_q[c] && q_ok[c];
                 v = vis ? v : -INFINITY;
                 sc[c][t][r] = v;
               }

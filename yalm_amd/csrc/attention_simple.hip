@@ -29,6 +29,7 @@ struct ScoreBias {
   float softcap;               // score <- softcap tanh(score / softcap) before the distance's term (0: no cap)
   const float* sink_logit;     // [heads]: one more term exp(sink_logit[head]) of the softmax's denominator, without a key (null: none)
   const float* slope;          // [heads]: -slope[head] * distance is added to every score (null: none)
+  int block;                   // a query sees the keys of its own block of `block` positions only (0: no blocks)
   __device__ __forceinline__ float at(int head, int distance) const {
     float term = table != nullptr ? table[(size_t)head * n + min(max(distance, 0), n - 1)] : 0.f;
     if (slope != nullptr) term -= slope[head] * (float)distance;
@@ -61,7 +62,7 @@ __global__ __launch_bounds__(WAVE) void attn_prefill_simple_kernel(
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int b = tok_seq[t], pos = tok_pos[t];
   const int g = h / (n_heads / n_kv_heads);
-  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int lo = first_visible(pos, window, sb.block);
   const float inv = sqrtf((float)hd);
   const size_t tile0 = (size_t)seq_tile0[b];
 
@@ -149,7 +150,7 @@ __global__ __launch_bounds__(WAVE) void attn_decode_simple_kernel(
 
   if (L > 0) {
     const int g = h / (n_heads / n_kv_heads);
-    const int lo = window > 0 ? max(0, L - window) : 0;       // first visible position
+    const int lo = first_visible(L - 1, window, sb.block);    // first visible position
     const int first_page = lo / PAGE, last_page = (L - 1) / PAGE;
     const int total = last_page - first_page + 1;
     const int per = (total + n_splits - 1) / n_splits;
@@ -337,12 +338,12 @@ extern "C" int yalm_attn_prefill_lse(const void* q, const void* k_stage, const v
                                  const int* tile_order, int n_order, int T, int B, int n_tiles, int n_heads,
                                  int n_kv_heads, int head_dim, int window, int dtype, int force_simple,
                                  const float* score_bias, int n_bias, float softcap, const float* sink_logit,
-                                 const float* slopes, hipStream_t stream) {
+                                 const float* slopes, int block, hipStream_t stream) {
   if (T <= 0) return YALM_OK;
-  if (bad_heads(n_heads, n_kv_heads, head_dim) || window < 0 || n_tiles <= 0) return YALM_ERR_ARG;
+  if (bad_heads(n_heads, n_kv_heads, head_dim) || window < 0 || block < 0 || n_tiles <= 0) return YALM_ERR_ARG;
   if ((score_bias != nullptr && n_bias <= 0) || softcap < 0.f) return YALM_ERR_ARG;
-  const ScoreBias sb = {score_bias, n_bias, softcap, sink_logit, slopes};
-  const ScoreShape shape = {score_bias, n_bias, softcap, sink_logit, slopes};
+  const ScoreBias sb = {score_bias, n_bias, softcap, sink_logit, slopes, block};
+  const ScoreShape shape = {score_bias, n_bias, softcap, sink_logit, slopes, block};
   dim3 grid(T, n_heads);
   if (dtype == YALM_F32) {
     if (head_dim <= ACC_SMALL * WAVE)
@@ -379,7 +380,7 @@ extern "C" int yalm_attn_prefill(const void* q, const void* k_stage, const void*
                                  hipStream_t stream) {
   return yalm_attn_prefill_lse(q, k_stage, v_stage, out, nullptr, nullptr, cu_seqlens, seq_tile0, tok_seq, tok_pos, tile_order,
                                n_order, T, B, n_tiles, n_heads, n_kv_heads, head_dim, window, dtype, force_simple,
-                               nullptr, 0, 0.f, nullptr, nullptr, stream);
+                               nullptr, 0, 0.f, nullptr, nullptr, 0, stream);
 }
 
 // merges the partial results of the splits (also used by the MFMA kernel)
@@ -406,12 +407,12 @@ int attn_decode_any(const void* q, const void* k_pages, const void* v_pages, con
                     int B, int n_heads, int n_kv_heads, int head_dim, int window, int n_splits, int n_pages,
                     int page_layout, int dtype, int force_simple, const SinkArgs& sinks, const int* step_max_len,
                     const int* seq_order, const float* score_bias, int n_bias, float softcap,
-                    const float* sink_logit, const float* slopes, hipStream_t stream) {
+                    const float* sink_logit, const float* slopes, int block, hipStream_t stream) {
   if (B <= 0) return YALM_OK;
-  const ScoreShape shape = {score_bias, n_bias, softcap, sink_logit, slopes};
-  if ((score_bias != nullptr && n_bias <= 0) || softcap < 0.f || (shape.any() && sinks.n_sinks > 0))
+  const ScoreShape shape = {score_bias, n_bias, softcap, sink_logit, slopes, block};
+  if ((score_bias != nullptr && n_bias <= 0) || softcap < 0.f || block < 0 || ((shape.any() || block > 0) && sinks.n_sinks > 0))
     return YALM_ERR_ARG;                                                // kept first positions are scored unshaped
-  const ScoreBias sb = {score_bias, n_bias, softcap, sink_logit, slopes};
+  const ScoreBias sb = {score_bias, n_bias, softcap, sink_logit, slopes, block};
   if (bad_heads(n_heads, n_kv_heads, head_dim) || window < 0 || n_splits <= 0 || ring_pages <= 0 ||
       !page_layout_ok(page_layout, head_dim))
     return YALM_ERR_ARG;
@@ -462,11 +463,11 @@ extern "C" int yalm_attn_decode_lse(const void* q, const void* k_pages, const vo
                                     int head_dim, int window, int n_splits, int n_pages, int page_layout, int dtype,
                                     int force_simple, const int* step_max_len, const int* seq_order,
                                     const float* score_bias, int n_bias, float softcap, const float* sink_logit,
-                                    const float* slopes, hipStream_t stream) {
+                                    const float* slopes, int block, hipStream_t stream) {
   SinkArgs none = {};
   return attn_decode_any(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len, out, lse,
                          partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout, dtype,
-                         force_simple, none, step_max_len, seq_order, score_bias, n_bias, softcap, sink_logit, slopes, stream);
+                         force_simple, none, step_max_len, seq_order, score_bias, n_bias, softcap, sink_logit, slopes, block, stream);
 }
 
 extern "C" int yalm_attn_decode(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
@@ -475,7 +476,7 @@ extern "C" int yalm_attn_decode(const void* q, const void* k_pages, const void* 
                                 int n_splits, int n_pages, int dtype, int force_simple, hipStream_t stream) {
   return yalm_attn_decode_lse(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len, out,
                               nullptr, partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages,
-                              YALM_PAGE_ROWS, dtype, force_simple, nullptr, nullptr, nullptr, 0, 0.f, nullptr, nullptr, stream);
+                              YALM_PAGE_ROWS, dtype, force_simple, nullptr, nullptr, nullptr, 0, 0.f, nullptr, nullptr, 0, stream);
 }
 
 extern "C" int yalm_attn_decode_sinks(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
@@ -511,7 +512,7 @@ extern "C" int yalm_attn_decode_sinks(const void* q, const void* k_pages, const 
   sk.n_sinks = n_sinks;
   return attn_decode_any(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len, out, nullptr,
                          partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout, dtype,
-                         force_simple, sk, step_max_len, seq_order, nullptr, 0, 0.f, nullptr, nullptr, stream);
+                         force_simple, sk, step_max_len, seq_order, nullptr, 0, 0.f, nullptr, nullptr, 0, stream);
 }
 
 // ---------------------------------------------------------------------------

@@ -16,10 +16,18 @@ struct ScoreShape {
   float softcap;
   const float* sink_logit;
   const float* slope;
+  int block;                  // part of the mask: a query sees the keys of its own block of `block` positions only (0: no blocks)
   __host__ __device__ bool any() const {
     return bias != nullptr || softcap > 0.f || sink_logit != nullptr || slope != nullptr;
   }
 };
+// The first position that a query at `pos` sees: not behind a window of `window` keys (0: none) and not before the start
+// of its own block of `block` positions, blocks counted from position 0 of the sequence (0: no blocks).
+__host__ __device__ __forceinline__ int first_visible(int pos, int window, int block) {
+  int lo = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
+  if (block > 0 && pos / block * block > lo) lo = pos / block * block;
+  return lo;
+}
 // cap tanh(s / cap) from the exponential instruction (the matrix-core kernels; absolute error about 1e-7 cap)
 __device__ __forceinline__ float soft_cap_fast(float s, float cap) {
   const float e = __builtin_amdgcn_exp2f(s * (2.0f * 1.4426950408889634f / cap));

@@ -170,17 +170,19 @@ long yalm_attn_decode_workspace(int B, int n_heads, int head_dim, int n_splits);
 // to which no key and no row of values belongs (scale, cap and distance term shape the keys' scores only; lse holds it).
 // slopes (device, float32 [n_heads]; may be null): -slopes[head] * distance is added to every score, as score_bias's
 // term is, without a table.
+// block (0: none): part of the mask; a query sees only the keys of its own block of `block` positions, blocks counted
+// from position 0 of the sequence (not together with attention sinks).
 int yalm_attn_prefill_lse(const void* q, const void* k_stage, const void* v_stage, void* out, float* out_f32, float* lse,
                           const int* cu_seqlens, const int* seq_tile0, const int* tok_seq, const int* tok_pos,
                           const int* tile_order, int n_order, int T, int B, int n_tiles, int n_heads, int n_kv_heads,
                           int head_dim, int window, int dtype, int force_simple, const float* score_bias, int n_bias,
-                          float softcap, const float* sink_logit, const float* slopes, hipStream_t stream);
+                          float softcap, const float* sink_logit, const float* slopes, int block, hipStream_t stream);
 int yalm_attn_decode_lse(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
                          int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
                          float* lse, float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
                          int n_splits, int n_pages, int page_layout, int dtype, int force_simple,
                          const int* step_max_len, const int* seq_order, const float* score_bias, int n_bias,
-                         float softcap, const float* sink_logit, const float* slopes, hipStream_t stream);
+                         float softcap, const float* sink_logit, const float* slopes, int block, hipStream_t stream);
 
 // Attention sinks beside a window (src/infer.cpp:305-319, 486-488): the first n_sinks positions of a
 // sequence stay visible when the window has moved past them, and each then counts as lying
@@ -347,6 +349,35 @@ int yalm_mlstm_chunks(const float* proj, const float* b_i, const float* b_f, con
                       float q_scale, float cap, float floor_, float eps, int n_slots, int chunk, int dtype,
                       hipStream_t stream);
 long yalm_mlstm_chunks_lds(int d, int chunk);
+
+// The gated delta rule with a decay per key channel, over the tokens of a step, float32 throughout.  H heads with values
+// of dv, Hq query/key heads of d (head h uses query/key head h / (H / Hq)).
+// proj float32 [T, 2 Hq d + H dv + H] = q | k | v | b: the projections before their short causal convolutions, and the step
+// size's logit.  low float32 [T, H d + H dv]: the decay's and the output gate's pre-activations.  conv_w float32
+// [2 Hq d + H dv, taps] (the last column is the current token's); decay_log [H], decay_bias [H d], w_norm [dv].
+// Per token: q, k, v <- silu(convolution); q, k <- unit vectors a head (x / sqrt(sum x^2 + unit_floor)), q times q_scale;
+// beta = sigmoid(b); g = exp(-exp(decay_log[h]) softplus(low + decay_bias)) per head and key channel; per head
+//   S <- diag(g) S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q;
+// out `dtype` [T, H dv] = o / rms(o over the head; eps) * w_norm * sigmoid(gate pre-activation).
+// state float32 [n_slots, H d dv + (2 Hq d + H dv) (taps - 1)]: S [H, d, dv], then the convolutions' last taps - 1 inputs
+// [channel, taps - 1] (the latest last); read and left advanced.  prep float32 [T, 2 Hq d + H dv + H + H d] and raw float32
+// [T, H dv]: scratch of the caller.  The tokens of sequence b are rows cu_seqlens[b] .. cu_seqlens[b + 1] - 1, in order;
+// tok_seq[t] is row t's sequence; seq_slot[b] < 0: a padding row, left alone (its output is zero).  d <= 256, taps <= 16.
+int yalm_gated_delta(const float* proj, const float* low, const float* conv_w, const float* decay_log,
+                     const float* decay_bias, const float* w_norm, float* state, float* prep, float* raw,
+                     const int* tok_seq, const int* cu_seqlens, const int* seq_slot, void* out, int T, int B, int H, int Hq,
+                     int d, int dv, int taps, float q_scale, float unit_floor, float eps, int n_slots, int dtype,
+                     hipStream_t stream);
+
+// x[t, :] = table[tokens[t], :] * scale + pos_table[positions[t], :] (both tables of `dtype`, [V, D] and [P, D]); a token
+// outside the vocabulary gives a row of zeros.
+int yalm_embed_learned(const void* table, const void* pos_table, int dtype, const int* tokens, const int* positions,
+                       float scale, float* out, int T, int D, int V, int P, hipStream_t stream);
+// out[i] = act(z[i]), out of `out_dtype`; kind 0: z/2 (1 + erf(z / sqrt 2)), 1: the tanh form of the same, 2: silu.
+int yalm_activate(const float* z, void* out, long n, int kind, int out_dtype, hipStream_t stream);
+// x[t, :] (+)= sigmoid(h[t, :] . w) * y[t, :]; h [T, D] and w [D] of `dtype`, x and y float32; accumulate 0: x is written.
+int yalm_gated_add(const float* y, const void* h, const void* w, int dtype, float* x, int T, int D, int accumulate,
+                   hipStream_t stream);
 
 // Yardsticks for the measurement (probes.hip): a kernel that only reads `bytes` bytes once with `workgroups`
 // workgroups (out: 1,024 words of scratch), and a loop of matrix-core instructions on registers (shape 32:

@@ -593,13 +593,17 @@ def _shape(softcap, sink_logit, n_heads, slopes=None):
 
 
 def attn_prefill(q, k_stage, v_stage, out, cu_seqlens, seq_tile0, tok_seq, tok_pos, n_heads, n_kv_heads, head_dim,
-                 window, tile_order=None, lse=None, out_f32=None, score_bias=None, softcap=0.0, sink_logit=None, slopes=None):
+                 window, tile_order=None, lse=None, out_f32=None, score_bias=None, softcap=0.0, sink_logit=None, slopes=None,
+                 block=0):
     """Causal (and windowed) attention of packed sequences that start at position 0, over
     the keys and values that rope_kv_write staged for this step.  tile_order (device int32,
     from prefill_tile_order) only changes the order of the work.  lse (float32 [T, n_heads], optional)
     receives the logarithm of every query's sum of exp(score), for attn_sink_mix; out_f32 (float32 [T, n_heads *
     head_dim], optional) the result before it is rounded to out's dtype, for the same.  score_bias: see _bias;
-    softcap, sink_logit: see _shape."""
+    softcap, sink_logit: see _shape.  block > 0: a query sees only the keys of its own block of `block` positions
+    (blocks counted from position 0 of its sequence), beside what the window says."""
+    if block < 0:
+        raise ValueError("a block of positions has a positive size (0: none)")
     _check_heads(n_heads, n_kv_heads, head_dim)
     T = q.shape[0]
     dt = q.dtype
@@ -623,7 +627,7 @@ def attn_prefill(q, k_stage, v_stage, out, cu_seqlens, seq_tile0, tok_seq, tok_p
                                                       T, B, n_tiles, n_heads, n_kv_heads, head_dim, int(window),
                                                       dtype_code(dt), 1 if FORCE_SIMPLE else 0,
                                                       *_bias(score_bias, n_heads), *_shape(softcap, sink_logit, n_heads, slopes),
-                                                      _stream()),
+                                                      int(block), _stream()),
                   "attn_prefill")
     return out
 
@@ -634,13 +638,13 @@ def attn_decode_workspace_floats(B, n_heads, head_dim, n_splits):
 
 def attn_decode(q, k_pages, v_pages, block_table, ring_pages, seq_slot, seq_len, out, partial, n_heads, n_kv_heads,
                 head_dim, window, n_splits, lse=None, sinks=None, layout=None, step_max_len=None, seq_order=None,
-                score_bias=None, softcap=0.0, sink_logit=None, slopes=None):
+                score_bias=None, softcap=0.0, sink_logit=None, slopes=None, block=0):
     """One query per sequence over the cache pages (laid out as `layout` says, default page_layout(head_dim));
     seq_len counts the new key.  lse as in attn_prefill.  step_max_len (int32 [1] on the device, optional): the
     length of the step's longest sequence, with which sequences of unequal lengths are cut into splits of equal
     size; seq_order (int32 [B] on the device, a permutation of the rows, optional): the order in which the
     workgroups take the rows (both change the division of the work and no result).  score_bias: see _bias; softcap,
-    sink_logit: see _shape (none of the three with sinks).
+    sink_logit: see _shape; block: see attn_prefill (none of these with sinks).
     sinks = (sink_k, sink_v [slots, n_kv_heads, n_sinks, head_dim], cos_sin or None, rotary_dim, store):
     the attention sinks that a query's window no longer covers are taken in where the splits are merged
     (their keys turned by max(0, position - window - n_sinks + 1) positions with the table cos_sin); with
@@ -671,11 +675,11 @@ def attn_decode(q, k_pages, v_pages, block_table, ring_pages, seq_slot, seq_len,
         library.check(library.lib().yalm_attn_decode_lse(
             p_q, p_kp, p_vp, p_bt, stride, ring_pages, p_ss, p_sl, p_o, p_lse, p_w, B, n_heads, n_kv_heads, head_dim,
             int(window), int(n_splits), n_pages, _layout(layout, head_dim), dtype_code(dt), force, p_max, p_ord,
-            *_bias(score_bias, n_heads), *_shape(softcap, sink_logit, n_heads, slopes), _stream()), "attn_decode")
+            *_bias(score_bias, n_heads), *_shape(softcap, sink_logit, n_heads, slopes), int(block), _stream()), "attn_decode")
         return out
     if lse is not None:
         raise ValueError("attn_decode leaves no lse when it takes the sinks in itself")
-    if score_bias is not None or softcap or sink_logit is not None or slopes is not None:
+    if score_bias is not None or softcap or sink_logit is not None or slopes is not None or block:
         raise ValueError("attention sinks are scored without a score bias, a cap or a sink logit: they do not go together")
     sink_k, sink_v, cos_sin, rotary_dim, store = sinks
     n_slots, _, n_sinks, _ = sink_k.shape
@@ -978,6 +982,81 @@ def mlstm_scan(proj, b_i, b_f, w_norm, state, cu_seqlens, seq_slot, out, n_heads
         _need(out, "out", None, (T, H * dv)), B, H, d, dv, float(q_scale), float(cap), float(floor), float(eps), n_slots,
         dtype_code(out.dtype), _stream()), "mlstm_scan")
     return out
+
+
+GATED_DELTA_MAX_KEY_DIM = 256     # a lane of the recurrence holds one column of a head's state in registers
+GATED_DELTA_MAX_TAPS = 16
+
+
+def gated_delta_state_elements(n_heads, n_qk_heads, d, dv, taps):
+    """Floats of per-sequence state that gated_delta keeps: the heads' matrices and the convolutions' last inputs."""
+    return n_heads * d * dv + (2 * n_qk_heads * d + n_heads * dv) * (taps - 1)
+
+
+def gated_delta(proj, low, conv_w, decay_log, decay_bias, w_norm, state, prep, raw, tok_seq, cu_seqlens, seq_slot, out,
+                n_heads, n_qk_heads, d, dv, taps, q_scale, unit_floor, eps):
+    """The gated delta rule with a decay per key channel over the tokens of a step, in float32.  proj float32
+    [T, 2 Hq d + H dv + H] = q | k | v | b (before the short causal convolutions conv_w [2 Hq d + H dv, taps], whose last column
+    is the current token's); low float32 [T, H d + H dv], the decay's and the output gate's pre-activations.  Per token:
+    q, k, v <- silu(convolution); q, k unit vectors a head (x / sqrt(sum x^2 + unit_floor)), q times q_scale; beta =
+    sigmoid(b); g = exp(-exp(decay_log[h]) softplus(low + decay_bias)); per head S <- diag(g) S, u = beta (v - S^T k),
+    S <- S + k u^T, o = S^T q; out [T, H dv] = o / rms(o) (a head at a time) * w_norm [dv] * sigmoid(gate pre-activation).
+    state float32 [slots, gated_delta_state_elements(...)] is read and left advanced; prep [T, 2 Hq d + H dv + H + H d] and raw
+    [T, H dv] are float32 scratch.  The tokens of sequence b are the rows cu_seqlens[b] .. cu_seqlens[b + 1] - 1; rows of
+    sequences with seq_slot < 0 are left alone."""
+    T = proj.shape[0]
+    B = seq_slot.shape[0]
+    H, Hq = n_heads, n_qk_heads
+    if not (0 < d <= GATED_DELTA_MAX_KEY_DIM and 0 < taps <= GATED_DELTA_MAX_TAPS and Hq > 0 and H % Hq == 0):
+        raise ValueError("gated_delta: key heads of %d, %d taps, %d heads on %d query heads are not offered" % (d, taps, H, Hq))
+    C = 2 * Hq * d + H * dv
+    if 2 * Hq * d * 4 > 64 * 1024:
+        raise ValueError("gated_delta: a token's queries and keys (%d numbers) are more than the kernel holds" % (2 * Hq * d))
+    n_slots = state.shape[0]
+    library.check(library.lib().yalm_gated_delta(
+        _need(proj, "proj", torch.float32, (T, C + H)), _need(low, "low", torch.float32, (T, H * d + H * dv)),
+        _need(conv_w, "conv_w", torch.float32, (C, taps)), _need(decay_log, "decay_log", torch.float32, (H,)),
+        _need(decay_bias, "decay_bias", torch.float32, (H * d,)), _need(w_norm, "w_norm", torch.float32, (dv,)),
+        _need(state, "state", torch.float32, (n_slots, gated_delta_state_elements(H, Hq, d, dv, taps))),
+        _need(prep, "prep", torch.float32, (T, C + H + H * d)), _need(raw, "raw", torch.float32, (T, H * dv)),
+        _need(tok_seq, "tok_seq", torch.int32, (T,)), _need(cu_seqlens, "cu_seqlens", torch.int32, (B + 1,)),
+        _need(seq_slot, "seq_slot", torch.int32, (B,)), _need(out, "out", None, (T, H * dv)), T, B, H, Hq, d, dv, taps,
+        float(q_scale), float(unit_floor), float(eps), n_slots, dtype_code(out.dtype), _stream()), "gated_delta")
+    return out
+
+
+def embed_learned(table, pos_table, tokens, positions, scale, out):
+    """out[t] = table[tokens[t]] * scale + pos_table[positions[t]] (float32 out; both tables of one dtype)."""
+    T = tokens.shape[0]
+    V, D = table.shape
+    P = pos_table.shape[0]
+    library.check(library.lib().yalm_embed_learned(
+        _need(table, "table", None, (V, D)), _need(pos_table, "pos_table", table.dtype, (P, D)), dtype_code(table.dtype),
+        _need(tokens, "tokens", torch.int32, (T,)), _need(positions, "positions", torch.int32, (T,)), float(scale),
+        _need(out, "out", torch.float32, (T, D)), T, D, V, P, _stream()), "embed_learned")
+    return out
+
+
+ACTIVATIONS = {"gelu_erf": 0, "gelu_tanh": 1, "silu": 2}
+
+
+def activate(z, out, kind):
+    """out = act(z), z float32, out of its own dtype and z's shape; kind: "gelu_erf" (z/2 (1 + erf(z / sqrt 2))),
+    "gelu_tanh" or "silu"."""
+    if kind not in ACTIVATIONS:
+        raise ValueError("activation %r is not offered (%s)" % (kind, ", ".join(ACTIVATIONS)))
+    library.check(library.lib().yalm_activate(_need(z, "z", torch.float32), _need(out, "out", None, tuple(z.shape)), z.numel(),
+                                              ACTIVATIONS[kind], dtype_code(out.dtype), _stream()), "activate")
+    return out
+
+
+def gated_add(y, h, w, x, accumulate=True):
+    """x[t] (+)= sigmoid(h[t] . w) * y[t]: a sublayer's result y (float32 [T, D]) under a gate of one number a token."""
+    T, D = y.shape
+    library.check(library.lib().yalm_gated_add(
+        _need(y, "y", torch.float32, (T, D)), _need(h, "h", None, (T, D)), _need(w, "w", h.dtype, (D,)), dtype_code(h.dtype),
+        _need(x, "x", torch.float32, (T, D)), T, D, 1 if accumulate else 0, _stream()), "gated_add")
+    return x
 
 
 # ---------------------------------------------------------------------------------------------------------------

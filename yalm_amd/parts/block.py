@@ -13,11 +13,13 @@ class PreNormResidualBlock(Part):
         p = layer_spec.prefix
         self.mixer_norm = build_part("norm", layer_spec.mixer_norm, dim, p)
         self.mixer = build_part("mixer", layer_spec.mixer, dim, p)
-        self.feed_forward_norm = build_part("norm", layer_spec.feed_forward_norm, dim, p)
-        self.feed_forward = build_part("feed_forward", layer_spec.feed_forward, dim, p)
+        self.feed_forward = self.feed_forward_norm = None             # a layer may have no feed-forward
+        if layer_spec.part("feed_forward") is not None:
+            self.feed_forward_norm = build_part("norm", layer_spec.feed_forward_norm, dim, p)
+            self.feed_forward = build_part("feed_forward", layer_spec.feed_forward, dim, p)
 
     def children(self):
-        return [self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward]
+        return [c for c in (self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward) if c is not None]
 
     def first_norm(self):
         """The norm that reads the residual stream first when this layer runs (the layer before
@@ -27,11 +29,13 @@ class PreNormResidualBlock(Part):
     def forward(self, x, ctx, line, writes_cache=True, next_norm=None):
         if self.mixer.fuses_norm(self.mixer_norm, x, ctx):
             self.mixer.forward_prenorm(x, self.mixer_norm, ctx, line, writes_cache,
-                                       emit_for=self.feed_forward_norm)
+                                       emit_for=self.feed_forward_norm if self.feed_forward is not None else next_norm)
         else:
             h = ctx.ws.get("block.h", (x.shape[0], self.dim), ctx.act_dtype)
             self.mixer_norm.forward(x, h, ctx)
             self.mixer.forward(h, x, ctx, line, writes_cache)
+        if self.feed_forward is None:
+            return
         if self.feed_forward.fuses_norm(self.feed_forward_norm, x, ctx):
             self.feed_forward.forward_prenorm(x, self.feed_forward_norm, ctx, emit_for=next_norm)
         else:

@@ -9,7 +9,8 @@ from .base import Part, part
 class TokenEmbedding(Part):
     """x[t] = float(table[token[t]]) (src/infer.cpp:454-475), times `scale` (default 1), plus, with `sinusoid_base` b,
     a position vector whose entry 2i is sin(p b^(-2i / width)) and whose entry 2i + 1 is the cosine of the same angle
-    (the frequencies are made in float64 and the angle is exact at every position)."""
+    (the frequencies are made in float64 and the angle is exact at every position), or, with `position_tensor` (a
+    tensor's name) and `n_positions`, plus the row of that learned table [n_positions, width] at the token's position."""
 
     def __init__(self, spec, dim, prefix):
         super().__init__(spec, dim, prefix)
@@ -17,14 +18,24 @@ class TokenEmbedding(Part):
         self.tensor = self.prefix + str(spec.params.get("tensor", "weight"))      # the table's name in a folder
         self.scale = float(spec.params.get("scale", 1.0))
         self.sinusoid_base = spec.params.get("sinusoid_base")
+        self.position_tensor = spec.params.get("position_tensor")
+        self.n_positions = int(spec.params.get("n_positions", 0) or 0)
+        if self.position_tensor and (self.sinusoid_base or self.n_positions <= 0):
+            raise ValueError("a learned position table needs n_positions, and goes without the sinusoid")
         self.table = None
         self.freq = None
+        self.positions = None
 
     def param_specs(self):
-        return [ParamSpec(self.tensor, (self.vocab_size, self.dim), init="embedding")]
+        out = [ParamSpec(self.tensor, (self.vocab_size, self.dim), init="embedding")]
+        if self.position_tensor:
+            out.append(ParamSpec(self.prefix + str(self.position_tensor), (self.n_positions, self.dim), init="embedding"))
+        return out
 
     def load(self, get, compute_dtype, device):
         self.table = place(get(self.tensor), compute_dtype, device)
+        if self.position_tensor:
+            self.positions = place(get(self.prefix + str(self.position_tensor)), compute_dtype, device)
         if self.sinusoid_base:
             import torch
             i = torch.arange((self.dim + 1) // 2, dtype=torch.float64)
@@ -32,9 +43,13 @@ class TokenEmbedding(Part):
             self.freq = torch.pow(base, -2.0 * i / self.dim).to(device)
 
     def weight_bytes(self):
-        return self.dim * self.table.element_size()          # one row per token
+        return (2 if self.positions is not None else 1) * self.dim * self.table.element_size()     # one row per token
 
     def forward(self, tokens, x, ctx):
+        if self.positions is not None:
+            if ctx.max_position >= self.n_positions:
+                raise ValueError("position %d is beyond the %d rows of the position table" % (ctx.max_position, self.n_positions))
+            return kernels.embed_learned(self.table, self.positions, tokens, ctx.tok_pos, self.scale, x)
         if self.freq is None and self.scale == 1.0:
             return kernels.embed(self.table, tokens, x)
         return kernels.embed_sinusoid(self.table, tokens, ctx.tok_pos, self.freq, self.scale, x)

@@ -1,6 +1,7 @@
 """RMSNorm: out = x * rsqrt(mean(x^2) + eps) * weight, sums in float32
 (src/infer.cpp:136-146, src/infer.cu:525-539).  The parameter `tensor` names the weight behind the
-part's prefix (default "weight").  `add_normed` is the norm of a layer that norms a sublayer's OUTPUT:
+part's prefix (default "weight"); with `offset` c the stored tensor is the weight's distance from c (weight = c +
+stored, formed in float32 and kept so, whatever the compute dtype: the sum has no bfloat16 of its own).  `add_normed` is the norm of a layer that norms a sublayer's OUTPUT:
 x += norm(y)."""
 import torch
 
@@ -15,13 +16,17 @@ class RMSNorm(Part):
         super().__init__(spec, dim, prefix)
         self.eps = float(spec.params["eps"])
         self.tensor = self.prefix + str(spec.params.get("tensor", "weight"))
+        self.offset = float(spec.params.get("offset", 0.0) or 0.0)
         self.weight = None
 
     def param_specs(self):
-        return [ParamSpec(self.tensor, (self.dim,), init="norm")]
+        return [ParamSpec(self.tensor, (self.dim,), init="norm_offset" if self.offset else "norm")]
 
     def load(self, get, compute_dtype, device):
-        self.weight = place(get(self.tensor), compute_dtype, device)
+        if self.offset:
+            self.weight = (get(self.tensor).to(torch.float32) + self.offset).to(device).contiguous()
+        else:
+            self.weight = place(get(self.tensor), compute_dtype, device)
         self.weight_f32 = self.weight if self.weight.dtype == torch.float32 else self.weight.float()
 
     def weight_bytes(self):

@@ -4,7 +4,9 @@ be left out.
 Per token: q, k, v = W h (+ biases); RMS norms over the WHOLE query and key projections (all heads at once, plain
 weights; `projection_norm`); the query times 1 + coef ln(floor((p + 1) / every) + 1) at position p (`q_temp`);
 score = (q . k) * scale, capped as cap tanh(score / cap) (`softcap`), plus the position part's term by the
-distance (a slope a head); a window; a softmax whose denominator also holds exp(sink_h), a learned logit a head
+distance (a slope a head); a window, and/or `block`: a query sees the keys of its own block of that many positions
+only, blocks counted from position 0 of the sequence (the cache then keeps a ring of a block's pages, as for a window
+of that width); a softmax whose denominator also holds exp(sink_h), a learned logit a head
 without key or value (`sink_logit`); the values of a layer with `value_blend` "later" are (1 - lam) v + lam v_first,
 v_first being the values that the layer with "first" made for the same token (lam a tensor), and the blended
 values are what the cache keeps.  Key and value heads may differ in size.
@@ -45,6 +47,9 @@ class ShapedAttention(Part):
         self.scale = float(p.get("scale") or self.key_dim ** -0.5)
         self.softcap = float(p.get("softcap") or 0.0)
         self.window = int(p.get("window", 0) or 0)
+        self.block = int(p.get("block", 0) or 0)
+        if self.window < 0 or self.block < 0:
+            raise ValueError("a window and a block of positions are positive (0: none)")
         self.q_temp = tuple(p["q_temp"]) if p.get("q_temp") else None
         self.projection_norm = bool(p.get("projection_norm", False))
         self.eps = float(p.get("eps", 1e-6))
@@ -110,7 +115,9 @@ class ShapedAttention(Part):
         return (self.wqkv.numel() + self.wo.numel()) * self.wqkv.element_size()
 
     def cache_request(self):
-        return KVRequest(self.n_kv_heads, self.pad, self.window, 0)
+        # a query inside a block sees fewer than `block` keys back: the ring of a window of that width holds them
+        reach = min(self.window, self.block) if self.window and self.block else (self.window or self.block)
+        return KVRequest(self.n_kv_heads, self.pad, reach, 0)
 
     def row_elements(self):
         return max(self.q_dim + self.k_dim + self.v_dim, self.n_heads * self.pad)
@@ -118,7 +125,7 @@ class ShapedAttention(Part):
     def describe(self, compute_dtype):
         what = "shaped attention, %d heads in %d groups, keys of %d and values of %d in heads of %d%s" % (
             self.n_heads, self.n_kv_heads, self.key_dim, self.value_dim, self.pad,
-            ", window %d" % self.window if self.window else "")
+            (", window %d" % self.window if self.window else "") + (", blocks of %d" % self.block if self.block else ""))
         if compute_dtype != torch.bfloat16:
             return what + ": float32-arithmetic kernels", False
         if self.pad in kernels.MFMA_HEAD_DIMS:
@@ -172,11 +179,12 @@ class ShapedAttention(Part):
         if prefill:
             kernels.attn_prefill(q, kst, vst, o, ctx.cu_seqlens, seq_tile0, ctx.tok_seq, ctx.tok_pos, H, G, P, self.window,
                                  tiles.get("tile_order"), score_bias=self.score_bias, softcap=self.softcap,
-                                 sink_logit=self.sink, slopes=self.slopes)
+                                 sink_logit=self.sink, slopes=self.slopes, block=self.block)
         else:
             n_splits = decode_splits(H, G, P, T, min(group.ring_pages, ctx.pages_bucket), ctx.ragged)
             partial = ws.get("attn.partial", (kernels.attn_decode_workspace_floats(T, H, P, n_splits),), torch.float32)
             kernels.attn_decode(q, k_pages, v_pages, group.table, group.ring_pages, ctx.seq_slot, ctx.seq_len, o, partial,
                                 H, G, P, self.window, n_splits, step_max_len=ctx.step_max_len, seq_order=ctx.seq_order,
-                                score_bias=self.score_bias, softcap=self.softcap, sink_logit=self.sink, slopes=self.slopes)
+                                score_bias=self.score_bias, softcap=self.softcap, sink_logit=self.sink, slopes=self.slopes,
+                                block=self.block)
         self._gemm(ctx, o, self.wo, x, kernels.EPI_ADD_F32)

@@ -71,6 +71,12 @@ def random_values(name, shape, init, fan_in, seed, device="cpu"):
         elif init == "embedding":
             u2 = _uniform01(key, start, n, 1, device)
             v = torch.sqrt(-2.0 * torch.log(u + (1.0 / (1 << 24)))) * torch.cos((2.0 * math.pi) * u2)
+        elif init == "norm_offset":          # a norm's weight stored as its distance from one
+            v = (u * 2.0 - 1.0) * 0.1
+        elif init == "decay_log":            # exp of it: the rate of a decay, 1/4 .. 4
+            v = (u * 2.0 - 1.0) * 1.3862943611198906
+        elif init == "taps":                 # a short convolution's weights
+            v = (u * 2.0 - 1.0) * 0.8
         elif init == "bias":
             v = (u * 2.0 - 1.0) * 0.5
         elif init == "fraction":
