@@ -8,7 +8,7 @@ shape with its window of 4,096 positions and prompts of 6,000 tokens).
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers N] [--dtype bf16|fp32] [--shape NAME]
                     [--prompt-len N] [--prefill-len N] [--batch B] [--points B,B] [--no-prefill]
                     [--kernels] [--ragged] [--sweep]
-    python bench.py --design situlorn|gedunex [--sizes 2048,4096] [--kernels] [--steps K] [--warmup W]
+    python bench.py --design situlorn|gedunex|bovozen [--sizes 2048,4096] [--kernels] [--steps K] [--warmup W]
 
 --kernels adds the time of every kernel of a decode step and of a prompt step, each taken alone at the
 shape's sizes (src/test.cpp:340-405 times single kernels so), with its rate against the peak;
@@ -20,7 +20,9 @@ Situlorn design (latent attention with and without a window, one layer on anothe
 mixture-of-experts feed-forwards) and four Llama layers of the same width and about the same weights, each a
 prompt of --prefill-len tokens and decode steps at --batch; with --kernels every kernel of both alone.  --design
 gedunex does the same for four layers of the Gedunex design (three shaped attentions under a window and one mLSTM,
-dense and mixture-of-experts feed-forwards) beside the Situlorn and the Llama layers.  The default workload and its
+dense and mixture-of-experts feed-forwards) beside the Situlorn and the Llama layers, --design bovozen for four layers
+of the Bovozen design (two gated delta rules, two attentions inside blocks of positions, a two-matrix feed-forward and
+mixtures of experts beside a shared expert) beside the Gedunex and the Llama layers.  The default workload and its
 line stay as they are.
 
 A step is one decode step as generation does it: the step function for a batch
@@ -113,8 +115,8 @@ KERNEL_FACES = ("embed", "rmsnorm", "gemm", "gemm_norm", "gemm_norm_qkv_rope", "
                 "gemm_chain", "gemm_chain_qkv_rope", "rope_kv_write", "rope_kv_write_tiles", "attn_prefill",
                 "attn_decode", "sink_store", "attn_sink_mix", "argmax", "cast", "norm_add", "polynorm", "head_matmul",
                 "latent_pack", "moe_route", "moe_select", "moe_pair_gate_up", "moe_pair_down", "moe_grouped", "embed_sinusoid",
-                "qkv_pack", "v_tiles", "mlstm_scan", "mlstm_chunks")
-FP32_FACES = ("mlstm_scan", "mlstm_chunks")     # kernels of float32 multiply-adds whatever the model's dtype: priced against that peak
+                "qkv_pack", "v_tiles", "mlstm_scan", "mlstm_chunks", "gated_delta", "embed_learned", "activate", "gated_add")
+FP32_FACES = ("mlstm_scan", "mlstm_chunks", "gated_delta")     # kernels of float32 multiply-adds whatever the model's dtype: priced against that peak
 
 
 def record_kernel_calls(run):
@@ -154,15 +156,17 @@ def kernel_cost(name, a, kw, kv_tokens, torch):
     if name == "attn_decode":
         q, kp = a[0], a[1]
         n_kv, hd = kp.shape[1], kp.shape[3]
+        if kw.get("block"):                     # a query reads the keys of its own block of positions only
+            kv_tokens = q.shape[0] * ((kv_tokens // max(q.shape[0], 1)) % kw["block"] + 1)
         return "attn_decode %d rows" % q.shape[0], 2 * kv_tokens * n_kv * hd * kp.element_size() + 2 * nbytes(q), \
             4.0 * q.shape[1] * kv_tokens
     if name == "attn_prefill":
         q, cu = a[0], a[4]
         lens = (cu[1:] - cu[:-1]).tolist()
         pairs = sum(n * (n + 1) // 2 for n in lens)
-        window = a[11]
-        if window:
-            pairs = sum(sum(min(i + 1, window) for i in range(n)) for n in lens)
+        window, block = a[11], kw.get("block", 0)
+        if window or block:
+            pairs = sum(sum(min(i + 1, window or i + 1, i % block + 1 if block else i + 1) for i in range(n)) for n in lens)
         return "attn_prefill %d tokens" % q.shape[0], nbytes(q, a[1], a[2], a[3]), 4.0 * q.shape[1] * pairs
     if name in ("rope_kv_write", "rope_kv_write_tiles"):
         q_out = a[1]
@@ -215,6 +219,19 @@ def kernel_cost(name, a, kw, kv_tokens, torch):
         # values, the query on the carried state and the token's share of the state's update
         per_token = 2.0 * d * min(chunk, max(T // B, 1)) / 2 + 2.0 * dv * min(chunk, max(T // B, 1)) / 2 + 4.0 * d * dv
         return "mlstm_chunks %d tokens" % T, nbytes(proj, out) + 2 * nbytes(a[5]) + 2 * B * H * (d * dv + d + 1) * 4, T * H * per_token
+    if name == "gated_delta":
+        proj, low, state, prep, raw, seq_slot, out = a[0], a[1], a[6], a[7], a[8], a[11], a[12]
+        H, d, dv = a[13], a[15], a[16]
+        T, B = proj.shape[0], seq_slot.shape[0]
+        # per token and head: the decay, S^T k, the rank-one update and S^T q, each over the d x dv state; the operands
+        # pass through memory twice (projections -> operands -> recurrence -> heads' norm), the state once each way
+        return "gated_delta %d tokens" % T, nbytes(proj, low, out) + 2 * nbytes(prep, raw) + 2 * B * H * d * dv * 4, 7.0 * T * H * d * dv
+    if name == "activate":
+        return "activate %dx%d" % tuple(a[0].shape), nbytes(a[0], a[1]), 0.0
+    if name == "gated_add":
+        return "gated_add %dx%d" % tuple(a[0].shape), nbytes(a[0], a[1]) + 2 * nbytes(a[3]), 0.0
+    if name == "embed_learned":
+        return "embed_learned %d" % a[2].shape[0], 2 * nbytes(a[5]), 0.0
     if name == "moe_route":
         return "moe_route %d tokens" % a[0].shape[0], nbytes(a[0], a[1]), 2.0 * a[0].shape[0] * a[1].numel()
     if name in ("moe_pair_gate_up", "moe_pair_down", "moe_grouped"):
@@ -319,6 +336,24 @@ def gedunex_config(width, n_layers=4):
             "embedding": {"scale": float(width) ** 0.5}, "layers": [pattern[i % 4] for i in range(n_layers)]}
 
 
+def bovozen_config(width, n_layers=4):
+    """Layers of the Bovozen design at a real model's sizes: delta-rule heads of 128 x 128 on half as many query/key heads
+    behind convolutions of four taps, low-rank products of width / 16; attention heads of 128 in groups of four inside
+    blocks of 1,536 positions (a prompt of 2,048 crosses one edge; a token decoded behind it sees the block's few hundred
+    keys); the feed-forwards of gedunex_config's sizes, the mixtures beside a shared expert of an expert's size."""
+    heads = width // 128
+    attn = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+            "mask": {"size": 1536}, "v_mix": True}
+    rec = {"heads": heads, "kv_heads": max(1, heads // 2), "dim": 128, "vdim": 128, "conv": 4, "decay_rank": width // 16,
+           "gate_rank": width // 16}
+    dense = {"kind": "dense", "ff": width * 21 // 4}               # two matrices: as many weights as a gated one of 3.5 width
+    moe = {"kind": "moe", "expert": {"ff": width // 2}, "router": {"experts": 32, "top": 4}, "shared": {"ff": width // 2}}
+    pattern = [{"type": "channel_delta", "mixer": rec, "mlp": dense}, {"type": "attention", "mixer": attn, "mlp": moe},
+               {"type": "attention", "mixer": attn, "mlp": moe}, {"type": "channel_delta", "mixer": rec, "mlp": moe}]
+    return {"architecture": "Bovozen", "vocab": 32000, "width": width, "norm": {"eps": 1e-5}, "max_positions": 8192,
+            "layers": [pattern[i % 4] for i in range(n_layers)]}
+
+
 def llama_config(width, n_layers=4):
     return {"architectures": ["LlamaForCausalLM"], "hidden_size": width, "intermediate_size": width * 7 // 2,
             "num_hidden_layers": n_layers, "num_attention_heads": width // 128, "num_key_value_heads": width // 512,
@@ -327,8 +362,8 @@ def llama_config(width, n_layers=4):
 
 
 def bench_design(args):
-    """Prompt and decode steps of the Situlorn design beside Llama layers of equal width, with every kernel alone on
-    request.  One JSON line."""
+    """Prompt and decode steps of a design's layers beside the closest design's and Llama layers of equal width, with
+    every kernel alone on request.  One JSON line."""
     import torch
     from yalm_amd import Engine, Model, Sampler
     dtype = {"bf16": torch.bfloat16, "fp32": torch.float32}[args.dtype]
@@ -337,8 +372,9 @@ def bench_design(args):
     sampler = Sampler(0)
     out = {}
     for width in [int(w) for w in args.sizes.split(",") if w]:
-        own = ("gedunex", gedunex_config(width)) if args.design == "gedunex" else ("situlorn", situlorn_config(width))
-        beside = (("situlorn", situlorn_config(width)),) if args.design == "gedunex" else ()
+        own = {"gedunex": gedunex_config, "situlorn": situlorn_config, "bovozen": bovozen_config}[args.design]
+        own = (args.design, own(width))
+        beside = {"gedunex": (("situlorn", situlorn_config(width)),), "bovozen": (("gedunex", gedunex_config(width)),)}.get(args.design, ())
         for design, cfg in (own,) + beside + (("llama", llama_config(width)),):
             model = Model.random(cfg, seed=0, dtype=dtype, device="cuda:0")
             V = model.vocab_size
@@ -442,7 +478,7 @@ def main():
     ap.add_argument("--context", type=int, default=0,
                     help="the reference's -T: past this many positions two attention sinks and the last "
                          "<context> - 2 positions are attended to (0: the shape's own window, if any)")
-    ap.add_argument("--design", default="", choices=["", "situlorn", "gedunex"],
+    ap.add_argument("--design", default="", choices=["", "situlorn", "gedunex", "bovozen"],
                     help="measure layers of this design beside Llama layers of equal width instead of the default workload")
     ap.add_argument("--sizes", default="2048,4096", help="widths for --design")
     args = ap.parse_args()

@@ -3,7 +3,7 @@
 // Per head a state S [d, dv]; per token, with unit vectors q (times q_scale) and k of the head's query/key head, values
 // v, a step size beta and decays g[i] in (0, 1) per key channel:
 //   S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q          (the read-out sees the token's own write)
-// Every column of S runs this on its own, so a lane owns one column, held in registers, and walks the tokens in order.
+// Every column of S runs this on its own, so four lanes own one column, held in registers, and walk the tokens in order.
 //
 // Three kernels a step: `prepare` turns a token's projections into the recurrence's operands (the short causal
 // convolutions with silu, the unit vectors, sigmoid and the decays), `carry` moves the convolutions' last inputs into
@@ -25,50 +25,61 @@ __device__ __forceinline__ float softplusf_(float z) { return z > 20.f ? z : log
 // prep [T, 2 Kq + Vv + H + H d]: q | k | v | beta | g, ready for the scan.
 // conv_w [2 Kq + Vv, taps], the last column is the current token's.  conv_state [n_slots, state_stride] holds, from
 // conv_off on, [channel][taps - 1] inputs of the tokens before this step, the latest last.
+// grid (T, units): a token's work is cut into units of at most 256 channels so that a step of few tokens still fills
+// the chip: unit u < 2 Hq is a query or key head (d <= 256: a thread a channel, the head's sum of squares across the
+// workgroup), the next ceil(Vv / 256) units are the values, the last ceil(H d / 256) the decays (the first of them also
+// the step sizes).
 __global__ __launch_bounds__(GD_THREADS) void gd_prepare_kernel(
     const float* __restrict__ proj, const float* __restrict__ low, const float* __restrict__ conv_w,
     const float* __restrict__ decay_log, const float* __restrict__ decay_bias, const float* __restrict__ state,
     const int* __restrict__ tok_seq, const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slot,
     float* __restrict__ prep, int H, int Hq, int d, int dv, int taps, float q_scale, float unit_floor, long state_stride,
     long conv_off) {
-  extern __shared__ float row[];                  // the token's q | k after convolution and silu
-  const int t = blockIdx.x;
+  __shared__ float part[GD_THREADS / WAVE];
+  const int t = blockIdx.x, unit = blockIdx.y, tid = threadIdx.x;
   const int Kq = Hq * d, Vv = H * dv, C = 2 * Kq + Vv;
   const int n_in = C + H, n_out = C + H + H * d;
+  const int v_units = (Vv + GD_THREADS - 1) / GD_THREADS;
   const int b = tok_seq[t];
   const int slot = seq_slot[b];
   float* out = prep + (size_t)t * n_out;
-  if (slot < 0) {                                 // a padding row
-    for (int i = threadIdx.x; i < n_out; i += GD_THREADS) out[i] = 0.f;
+  const float* x = proj + (size_t)t * n_in;
+  if (unit >= 2 * Hq + v_units) {                 // decays (and step sizes)
+    const int du = unit - 2 * Hq - v_units, i = du * GD_THREADS + tid;
+    if (du == 0)
+      for (int h = tid; h < H; h += GD_THREADS) out[C + h] = slot < 0 ? 0.f : sigmoidf_(x[C + h]);
+    if (i < H * d) {
+      const float z = low[(size_t)t * (H * d + Vv) + i];
+      out[C + H + i] = slot < 0 ? 0.f : expf(-expf(decay_log[i / d]) * softplusf_(z + decay_bias[i]));
+    }
     return;
   }
-  const int p = t - cu_seqlens[b];                // the token's place among its sequence's tokens of this step
-  const float* x = proj + (size_t)t * n_in;
-  const float* held = state + (size_t)slot * state_stride + conv_off;
-  for (int c = threadIdx.x; c < C; c += GD_THREADS) {
+  const bool head = unit < 2 * Hq;
+  const int c = head ? unit * d + tid : 2 * Kq + (unit - 2 * Hq) * GD_THREADS + tid;
+  const bool live = head ? tid < d : c < C;
+  float a = 0.f;
+  if (live && slot >= 0) {
+    const int p = t - cu_seqlens[b];              // the token's place among its sequence's tokens of this step
+    const float* held = state + (size_t)slot * state_stride + conv_off;
     const float* w = conv_w + (size_t)c * taps;
     float acc = w[taps - 1] * x[c];
     for (int back = 1; back < taps; ++back) {
       const float past = back <= p ? proj[(size_t)(t - back) * n_in + c] : held[(size_t)c * (taps - 1) + (taps - 1 - back + p)];
       acc = fmaf(w[taps - 1 - back], past, acc);
     }
-    const float a = acc / (1.0f + expf(-acc));
-    if (c < 2 * Kq) row[c] = a; else out[c] = a;
+    a = acc / (1.0f + expf(-acc));
   }
+  if (!head) {
+    if (live) out[c] = a;
+    return;
+  }
+  const float ss = wave_sum(a * a);               // unit vectors: the head's sum of squares across the workgroup
+  if (tid % WAVE == 0) part[tid / WAVE] = ss;
   __syncthreads();
-  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-  for (int hh = wave; hh < 2 * Hq; hh += GD_THREADS / WAVE) {         // unit vectors, a head a wave
-    const float* r = row + (size_t)hh * d;
-    float ss = 0.f;
-    for (int i = lane; i < d; i += WAVE) ss = fmaf(r[i], r[i], ss);
-    ss = wave_sum(ss);
-    const float s = (hh < Hq ? q_scale : 1.0f) / sqrtf(ss + unit_floor);
-    for (int i = lane; i < d; i += WAVE) out[(size_t)hh * d + i] = r[i] * s;
-  }
-  for (int h = threadIdx.x; h < H; h += GD_THREADS) out[C + h] = sigmoidf_(x[C + h]);
-  const float* z = low + (size_t)t * (H * d + Vv);
-  for (int i = threadIdx.x; i < H * d; i += GD_THREADS)
-    out[C + H + i] = expf(-expf(decay_log[i / d]) * softplusf_(z[i] + decay_bias[i]));
+  float total = 0.f;
+#pragma unroll
+  for (int w = 0; w < GD_THREADS / WAVE; ++w) total += part[w];
+  if (live) out[c] = slot < 0 ? 0.f : a * ((unit < Hq ? q_scale : 1.0f) / sqrtf(total + unit_floor));
 }
 
 // The convolutions' inputs that the next step needs: the last taps - 1 of (what was held) ++ (this step's).
@@ -84,15 +95,29 @@ __global__ void gd_carry_kernel(const float* __restrict__ proj, float* __restric
     held[i] = n + i < m ? held[n + i] : proj[(size_t)(t0 + n + i - m) * n_in + c];
 }
 
-// grid (columns / 64, H, B), one wave: lane j owns column j0 + j of head h of sequence b.
-template <int D>
+// grid (columns / 16, H, B), one wave: lane (c, r) = (lane / 4, lane % 4) owns the rows r DR .. r DR + DR - 1 of column
+// j0 + c of head h of sequence b, in registers; the two sums over a column's rows (S^T k and S^T q) are finished across
+// the four neighbouring lanes of a column with two permutes inside the quad (no LDS).  A prompt of one sequence so keeps
+// dv / 16 waves a head busy, and a token costs a lane 4 DR multiply-adds in a row instead of 4 d.
+constexpr int GD_COLS = 16, GD_ROWS = WAVE / GD_COLS;
+static_assert(GD_ROWS == 4, "quad_sum adds over four neighbouring lanes");
+
+__device__ __forceinline__ float quad_sum(float x) {
+  const float y = x + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, x), 0xB1, 0xF, 0xF, true));
+  return y + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, y), 0x4E, 0xF, 0xF, true));
+}
+
+template <int DR>
 __global__ __launch_bounds__(WAVE) void gd_scan_kernel(const float* __restrict__ prep, float* __restrict__ state,
                                                        const int* __restrict__ cu_seqlens,
                                                        const int* __restrict__ seq_slot, float* __restrict__ raw, int H,
                                                        int Hq, int d, int dv, long state_stride) {
-  __shared__ __attribute__((aligned(16))) float sq[GD_TOKENS][D], sk[GD_TOKENS][D], sg[GD_TOKENS][D];
-  __shared__ float sv[GD_TOKENS][WAVE], sb[GD_TOKENS];
-  const int b = blockIdx.z, h = blockIdx.y, lane = threadIdx.x, j = blockIdx.x * WAVE + lane;
+  constexpr int LD = DR + 4;             // a row group's operands start 4 banks further on than the one's before
+  __shared__ __attribute__((aligned(16))) float sq[GD_TOKENS][GD_ROWS * LD], sk[GD_TOKENS][GD_ROWS * LD],
+      sg[GD_TOKENS][GD_ROWS * LD];
+  __shared__ float sv[GD_TOKENS][GD_COLS], sb[GD_TOKENS];
+  const int b = blockIdx.z, h = blockIdx.y, lane = threadIdx.x;
+  const int c = lane / GD_ROWS, r = lane % GD_ROWS, j = blockIdx.x * GD_COLS + c;
   const int slot = seq_slot[b];
   if (slot < 0) return;
   const int t0 = cu_seqlens[b], t1 = cu_seqlens[b + 1];
@@ -100,45 +125,85 @@ __global__ __launch_bounds__(WAVE) void gd_scan_kernel(const float* __restrict__
   const int Kq = Hq * d, Vv = H * dv, C = 2 * Kq + Vv, n_out = C + H + H * d;
   const int hq = h / (H / Hq);
   const bool live = j < dv;
+  const int i0 = r * DR;
   float* col = state + (size_t)slot * state_stride + ((size_t)h * d) * dv + (live ? j : 0);
-  float S[D];
+  float S[DR];
 #pragma unroll
-  for (int i = 0; i < D; ++i) S[i] = live && i < d ? col[(size_t)i * dv] : 0.f;
+  for (int i = 0; i < DR; ++i) S[i] = live && i0 + i < d ? col[(size_t)(i0 + i) * dv] : 0.f;
+  // The operands of GD_TOKENS tokens wait in LDS; those of the next GD_TOKENS are asked for before the recurrence walks
+  // the ones at hand and rest in registers meanwhile, so that memory's latency is paid once a sequence, not once a group.
+  constexpr int NLD = GD_TOKENS * GD_ROWS * DR / WAVE, NV = GD_TOKENS * GD_COLS / WAVE;
+  static_assert(GD_TOKENS * GD_ROWS * DR % WAVE == 0 && GD_TOKENS * GD_COLS % WAVE == 0 && GD_TOKENS <= WAVE, "whole rounds of loads");
+  float pq[NLD], pk[NLD], pg[NLD], pv[NV], pb;
+  auto fetch = [&](int c0) {
+    const int n = min(GD_TOKENS, t1 - c0);
+#pragma unroll
+    for (int k = 0; k < NLD; ++k) {
+      const int idx = k * WAVE + lane, tt = idx / (GD_ROWS * DR), i = idx % (GD_ROWS * DR);
+      const bool in = tt < n && i < d;
+      const float* row = prep + (size_t)(c0 + (in ? tt : 0)) * n_out + (in ? i : 0);
+      pq[k] = in ? row[hq * d] : 0.f;
+      pk[k] = in ? row[Kq + hq * d] : 0.f;
+      pg[k] = in ? row[C + H + h * d] : 0.f;
+    }
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int idx = k * WAVE + lane, tt = idx / GD_COLS, jj = blockIdx.x * GD_COLS + idx % GD_COLS;
+      pv[k] = tt < n && jj < dv ? prep[(size_t)(c0 + tt) * n_out + 2 * Kq + h * dv + jj] : 0.f;
+    }
+    pb = lane < n ? prep[(size_t)(c0 + lane) * n_out + C + h] : 0.f;
+  };
+  fetch(t0);
   for (int c0 = t0; c0 < t1; c0 += GD_TOKENS) {
     const int n = min(GD_TOKENS, t1 - c0);
     __syncthreads();
-    for (int idx = lane; idx < n * D; idx += WAVE) {
-      const int tt = idx / D, i = idx % D;
-      const float* r = prep + (size_t)(c0 + tt) * n_out;
-      const bool in = i < d;
-      sq[tt][i] = in ? r[hq * d + i] : 0.f;
-      sk[tt][i] = in ? r[Kq + hq * d + i] : 0.f;
-      sg[tt][i] = in ? r[C + H + h * d + i] : 0.f;
+#pragma unroll
+    for (int k = 0; k < NLD; ++k) {
+      const int idx = k * WAVE + lane, tt = idx / (GD_ROWS * DR), i = idx % (GD_ROWS * DR);
+      const int at = (i / DR) * LD + i % DR;
+      sq[tt][at] = pq[k];
+      sk[tt][at] = pk[k];
+      sg[tt][at] = pg[k];
     }
-    for (int tt = 0; tt < n; ++tt) sv[tt][lane] = live ? prep[(size_t)(c0 + tt) * n_out + 2 * Kq + h * dv + j] : 0.f;
-    if (lane < n) sb[lane] = prep[(size_t)(c0 + lane) * n_out + C + h];
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int idx = k * WAVE + lane;
+      sv[idx / GD_COLS][idx % GD_COLS] = pv[k];
+    }
+    if (lane < GD_TOKENS) sb[lane] = pb;
     __syncthreads();
+    if (c0 + GD_TOKENS < t1) fetch(c0 + GD_TOKENS);
+#pragma unroll 2
     for (int tt = 0; tt < n; ++tt) {
-      float kv = 0.f;
+      const float* gk = &sg[tt][r * LD];
+      const float* kk = &sk[tt][r * LD];
+      const float* qq = &sq[tt][r * LD];
+      float kv0 = 0.f, kv1 = 0.f;
 #pragma unroll
-      for (int i = 0; i < D; ++i) {
-        S[i] *= sg[tt][i];
-        kv = fmaf(S[i], sk[tt][i], kv);
+      for (int i = 0; i < DR; i += 2) {
+        S[i] *= gk[i];
+        S[i + 1] *= gk[i + 1];
+        kv0 = fmaf(S[i], kk[i], kv0);
+        kv1 = fmaf(S[i + 1], kk[i + 1], kv1);
       }
-      const float u = sb[tt] * (sv[tt][lane] - kv);
-      float o = 0.f;
+      const float kv = quad_sum(kv0 + kv1);
+      const float u = sb[tt] * (sv[tt][c] - kv);
+      float o0 = 0.f, o1 = 0.f;
 #pragma unroll
-      for (int i = 0; i < D; ++i) {
-        S[i] = fmaf(sk[tt][i], u, S[i]);
-        o = fmaf(S[i], sq[tt][i], o);
+      for (int i = 0; i < DR; i += 2) {
+        S[i] = fmaf(kk[i], u, S[i]);
+        S[i + 1] = fmaf(kk[i + 1], u, S[i + 1]);
+        o0 = fmaf(S[i], qq[i], o0);
+        o1 = fmaf(S[i + 1], qq[i + 1], o1);
       }
-      if (live) raw[(size_t)(c0 + tt) * Vv + h * dv + j] = o;
+      const float o = quad_sum(o0 + o1);
+      if (live && r == 0) raw[(size_t)(c0 + tt) * Vv + h * dv + j] = o;
     }
   }
   if (live) {
 #pragma unroll
-    for (int i = 0; i < D; ++i)
-      if (i < d) col[(size_t)i * dv] = S[i];
+    for (int i = 0; i < DR; ++i)
+      if (i0 + i < d) col[(size_t)(i0 + i) * dv] = S[i];
   }
 }
 
@@ -178,9 +243,9 @@ extern "C" int yalm_gated_delta(const float* proj, const float* low, const float
   if (dtype != YALM_F32 && dtype != YALM_BF16) return YALM_ERR_DTYPE;
   const int Kq = Hq * d, C = 2 * Kq + H * dv;
   const long conv_off = (long)H * d * dv, state_stride = conv_off + (long)C * (taps - 1);
-  const size_t lds = (size_t)2 * Kq * sizeof(float);
-  if (lds > 64 * 1024) return YALM_ERR_ARG;
-  gd_prepare_kernel<<<T, GD_THREADS, lds, stream>>>(proj, low, conv_w, decay_log, decay_bias, state, tok_seq, cu_seqlens,
+  const int units = 2 * Hq + ceil_div(H * dv, GD_THREADS) + ceil_div(H * d, GD_THREADS);
+  if (units > 65535 || d > GD_THREADS) return YALM_ERR_ARG;
+  gd_prepare_kernel<<<dim3(T, units), GD_THREADS, 0, stream>>>(proj, low, conv_w, decay_log, decay_bias, state, tok_seq, cu_seqlens,
                                                     seq_slot, prep, H, Hq, d, dv, taps, q_scale, unit_floor, state_stride,
                                                     conv_off);
   if (int rc = launch_status(); rc != YALM_OK) return rc;
@@ -189,13 +254,15 @@ extern "C" int yalm_gated_delta(const float* proj, const float* low, const float
                                                                    state_stride, conv_off);
     if (int rc = launch_status(); rc != YALM_OK) return rc;
   }
-  const dim3 grid(ceil_div(dv, WAVE), H, B);
-#define GD_SCAN(D) gd_scan_kernel<D><<<grid, WAVE, 0, stream>>>(prep, state, cu_seqlens, seq_slot, raw, H, Hq, d, dv, state_stride)
-  if (d <= 16) GD_SCAN(16);
-  else if (d <= 32) GD_SCAN(32);
-  else if (d <= 64) GD_SCAN(64);
-  else if (d <= 128) GD_SCAN(128);
-  else GD_SCAN(256);
+  if (ceil_div(dv, GD_COLS) > 65535) return YALM_ERR_ARG;
+  const dim3 grid(ceil_div(dv, GD_COLS), H, B);
+#define GD_SCAN(DR) gd_scan_kernel<DR><<<grid, WAVE, 0, stream>>>(prep, state, cu_seqlens, seq_slot, raw, H, Hq, d, dv, state_stride)
+  if (d <= 8) GD_SCAN(2);                 // rows a lane: a quarter of the key head, rounded up to the next template
+  else if (d <= 16) GD_SCAN(4);
+  else if (d <= 32) GD_SCAN(8);
+  else if (d <= 64) GD_SCAN(16);
+  else if (d <= 128) GD_SCAN(32);
+  else GD_SCAN(64);
 #undef GD_SCAN
   if (int rc = launch_status(); rc != YALM_OK) return rc;
   if (dtype == YALM_F32)

@@ -1010,8 +1010,8 @@ def gated_delta(proj, low, conv_w, decay_log, decay_bias, w_norm, state, prep, r
     if not (0 < d <= GATED_DELTA_MAX_KEY_DIM and 0 < taps <= GATED_DELTA_MAX_TAPS and Hq > 0 and H % Hq == 0):
         raise ValueError("gated_delta: key heads of %d, %d taps, %d heads on %d query heads are not offered" % (d, taps, H, Hq))
     C = 2 * Hq * d + H * dv
-    if 2 * Hq * d * 4 > 64 * 1024:
-        raise ValueError("gated_delta: a token's queries and keys (%d numbers) are more than the kernel holds" % (2 * Hq * d))
+    if 2 * Hq + (H * dv + 255) // 256 + (H * d + 255) // 256 > 65535:
+        raise ValueError("gated_delta: %d heads of %d x %d are more than a launch's grid holds" % (H, d, dv))
     n_slots = state.shape[0]
     library.check(library.lib().yalm_gated_delta(
         _need(proj, "proj", torch.float32, (T, C + H)), _need(low, "low", torch.float32, (T, H * d + H * dv)),

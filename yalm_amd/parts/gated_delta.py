@@ -108,7 +108,7 @@ class GatedDelta(Part):
         return self.channels + self.n_heads + self.gk
 
     def describe(self, compute_dtype):
-        return "gated delta rule, %d heads of %d x %d on %d query heads, %d taps: a state column a lane, float32" % (
+        return "gated delta rule, %d heads of %d x %d on %d query heads, %d taps: a state column in the registers of four lanes, float32" % (
             self.n_heads, self.key_dim, self.value_dim, self.n_qk_heads, self.taps), False
 
     def forward(self, h, x, ctx, line, writes_cache=True):
