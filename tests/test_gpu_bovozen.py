@@ -82,15 +82,17 @@ def test_gate_of_one_number_a_token(T, D, dtype, accumulate):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n_first", [50, 80])
 @pytest.mark.parametrize("H,G,d,dv,taps", [(1, 1, 4, 4, 2), (4, 2, 8, 12, 4), (6, 2, 3, 5, 1), (2, 2, 32, 32, 3), (1, 1, 64, 200, 5),
                                            (3, 1, 20, 7, 2), (2, 1, 128, 70, 3), (1, 1, 200, 9, 16)])
-def test_delta_rule_kernel(dtype, H, G, d, dv, taps):
+def test_delta_rule_kernel(dtype, H, G, d, dv, taps, n_first):
     """Two sequences and a padding row: the first pieces of the texts as a step of whole prompts (one shorter than the
     convolution, one of many tokens), then single tokens, against the plain recurrence over the whole texts; the state
-    and the convolutions' inputs left behind against the plain ones."""
+    and the convolutions' inputs left behind against the plain ones.  The two lengths of the first piece fall on either
+    side of the step size from which the recurrence's kernel spreads a state column over eight lanes instead of four."""
     from yalm_amd.ops import kernels
     D = 24
-    lens = [57, 9]
+    lens = [n_first + 7, 9]
     g = gen(H * 100 + d)
     rn = lambda *s, sc=1.0: torch.randn(*s, generator=g, dtype=F64) * sc
     ra, rg = 3, 2
@@ -122,7 +124,7 @@ def test_delta_rule_kernel(dtype, H, G, d, dv, taps):
                             i32(tok_seq), i32(cu), i32(seq_slot), out, H, G, d, dv, taps, d ** -0.5, P.UNIT_FLOOR, 1e-5)
         return out.float().cpu().to(F64)
 
-    first = [50, 1]                                # the second prompt is shorter than most of the convolutions
+    first = [n_first, 1]                           # the second prompt is shorter than most of the convolutions
     got = [[], []]
     out = step([hs[0][:first[0]], hs[1][:first[1]]], [0, first[0], first[0] + first[1]], slots)
     got[0].append(out[:first[0]]); got[1].append(out[first[0]:])

@@ -95,23 +95,29 @@ __global__ void gd_carry_kernel(const float* __restrict__ proj, float* __restric
     held[i] = n + i < m ? held[n + i] : proj[(size_t)(t0 + n + i - m) * n_in + c];
 }
 
-// grid (columns / 16, H, B), one wave: lane (c, r) = (lane / 4, lane % 4) owns the rows r DR .. r DR + DR - 1 of column
-// j0 + c of head h of sequence b, in registers; the two sums over a column's rows (S^T k and S^T q) are finished across
-// the four neighbouring lanes of a column with two permutes inside the quad (no LDS).  A prompt of one sequence so keeps
-// dv / 16 waves a head busy, and a token costs a lane 4 DR multiply-adds in a row instead of 4 d.
-constexpr int GD_COLS = 16, GD_ROWS = WAVE / GD_COLS;
-static_assert(GD_ROWS == 4, "quad_sum adds over four neighbouring lanes");
-
-__device__ __forceinline__ float quad_sum(float x) {
-  const float y = x + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, x), 0xB1, 0xF, 0xF, true));
-  return y + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, y), 0x4E, 0xF, 0xF, true));
+// grid (columns / GD_COLS, H, B), one wave: lane (c, r) = (lane / GD_ROWS, lane % GD_ROWS) owns the rows r DR .. r DR + DR - 1
+// of column j0 + c of head h of sequence b, in registers; the two sums over a column's rows (S^T k and S^T q) are
+// finished across the GD_ROWS neighbouring lanes of a column with permutes inside a row of 16 lanes (no LDS).  With
+// eight lanes a column a prompt of one sequence keeps dv / 8 waves a head busy and a token costs a lane 4 DR = d / 2
+// multiply-adds in a row; with four lanes a column (steps of single tokens) a lane's 16 columns are 64 bytes of a
+// state's row, which is what the state's way from and to memory likes.
+template <int ROWS>
+__device__ __forceinline__ float rows_sum(float x) {
+  static_assert(ROWS == 4 || ROWS == 8, "sums over four or eight neighbouring lanes");
+  x += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, x), 0xB1, 0xF, 0xF, true));   // lanes 1 0 3 2
+  x += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, x), 0x4E, 0xF, 0xF, true));   // lanes 2 3 0 1
+  if constexpr (ROWS == 8)                        // every lane of a quad holds the quad's sum: lane 7 - i has the other quad's
+    x += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, x), 0x141, 0xF, 0xF, true));
+  return x;
 }
 
-template <int DR>
+template <int DR, int GD_ROWS>
 __global__ __launch_bounds__(WAVE) void gd_scan_kernel(const float* __restrict__ prep, float* __restrict__ state,
                                                        const int* __restrict__ cu_seqlens,
                                                        const int* __restrict__ seq_slot, float* __restrict__ raw, int H,
                                                        int Hq, int d, int dv, long state_stride) {
+  static_assert(DR % 4 == 0, "a lane reads its rows' operands four at a time");
+  constexpr int GD_COLS = WAVE / GD_ROWS;
   constexpr int LD = DR + 4;             // a row group's operands start 4 banks further on than the one's before
   __shared__ __attribute__((aligned(16))) float sq[GD_TOKENS][GD_ROWS * LD], sk[GD_TOKENS][GD_ROWS * LD],
       sg[GD_TOKENS][GD_ROWS * LD];
@@ -175,28 +181,40 @@ __global__ __launch_bounds__(WAVE) void gd_scan_kernel(const float* __restrict__
     if (c0 + GD_TOKENS < t1) fetch(c0 + GD_TOKENS);
 #pragma unroll 2
     for (int tt = 0; tt < n; ++tt) {
-      const float* gk = &sg[tt][r * LD];
-      const float* kk = &sk[tt][r * LD];
-      const float* qq = &sq[tt][r * LD];
-      float kv0 = 0.f, kv1 = 0.f;
+      // the token's operands for this lane's rows, four at a time (a row group starts on a 16-byte border)
+      const float4* g4 = reinterpret_cast<const float4*>(&sg[tt][r * LD]);
+      const float4* k4 = reinterpret_cast<const float4*>(&sk[tt][r * LD]);
+      const float4* q4 = reinterpret_cast<const float4*>(&sq[tt][r * LD]);
+      float kk[DR];
+      float kv0 = 0.f, kv1 = 0.f, kv2 = 0.f, kv3 = 0.f;
 #pragma unroll
-      for (int i = 0; i < DR; i += 2) {
-        S[i] *= gk[i];
-        S[i + 1] *= gk[i + 1];
-        kv0 = fmaf(S[i], kk[i], kv0);
-        kv1 = fmaf(S[i + 1], kk[i + 1], kv1);
+      for (int v = 0; v < DR / 4; ++v) {
+        const float4 g = g4[v], k = k4[v];
+        const int i = 4 * v;
+        kk[i] = k.x, kk[i + 1] = k.y, kk[i + 2] = k.z, kk[i + 3] = k.w;
+        S[i] *= g.x, S[i + 1] *= g.y, S[i + 2] *= g.z, S[i + 3] *= g.w;
+        kv0 = fmaf(S[i], k.x, kv0);
+        kv1 = fmaf(S[i + 1], k.y, kv1);
+        kv2 = fmaf(S[i + 2], k.z, kv2);
+        kv3 = fmaf(S[i + 3], k.w, kv3);
       }
-      const float kv = quad_sum(kv0 + kv1);
+      const float kv = rows_sum<GD_ROWS>((kv0 + kv1) + (kv2 + kv3));
       const float u = sb[tt] * (sv[tt][c] - kv);
-      float o0 = 0.f, o1 = 0.f;
+      float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
 #pragma unroll
-      for (int i = 0; i < DR; i += 2) {
+      for (int v = 0; v < DR / 4; ++v) {
+        const float4 q = q4[v];
+        const int i = 4 * v;
         S[i] = fmaf(kk[i], u, S[i]);
         S[i + 1] = fmaf(kk[i + 1], u, S[i + 1]);
-        o0 = fmaf(S[i], qq[i], o0);
-        o1 = fmaf(S[i + 1], qq[i + 1], o1);
+        S[i + 2] = fmaf(kk[i + 2], u, S[i + 2]);
+        S[i + 3] = fmaf(kk[i + 3], u, S[i + 3]);
+        o0 = fmaf(S[i], q.x, o0);
+        o1 = fmaf(S[i + 1], q.y, o1);
+        o2 = fmaf(S[i + 2], q.z, o2);
+        o3 = fmaf(S[i + 3], q.w, o3);
       }
-      const float o = quad_sum(o0 + o1);
+      const float o = rows_sum<GD_ROWS>((o0 + o1) + (o2 + o3));
       if (live && r == 0) raw[(size_t)(c0 + tt) * Vv + h * dv + j] = o;
     }
   }
@@ -254,15 +272,25 @@ extern "C" int yalm_gated_delta(const float* proj, const float* low, const float
                                                                    state_stride, conv_off);
     if (int rc = launch_status(); rc != YALM_OK) return rc;
   }
-  if (ceil_div(dv, GD_COLS) > 65535) return YALM_ERR_ARG;
-  const dim3 grid(ceil_div(dv, GD_COLS), H, B);
-#define GD_SCAN(DR) gd_scan_kernel<DR><<<grid, WAVE, 0, stream>>>(prep, state, cu_seqlens, seq_slot, raw, H, Hq, d, dv, state_stride)
-  if (d <= 8) GD_SCAN(2);                 // rows a lane: a quarter of the key head, rounded up to the next template
-  else if (d <= 16) GD_SCAN(4);
-  else if (d <= 32) GD_SCAN(8);
-  else if (d <= 64) GD_SCAN(16);
-  else if (d <= 128) GD_SCAN(32);
-  else GD_SCAN(64);
+  // steps of prompts: eight lanes a column; steps of few tokens a sequence: four
+  const bool wide = T >= 32 * B && d > 16;
+  const int cols = WAVE / (wide ? 8 : 4);
+  if (ceil_div(dv, cols) > 65535) return YALM_ERR_ARG;
+  const dim3 grid(ceil_div(dv, cols), H, B);
+#define GD_SCAN(DR, ROWS) \
+  gd_scan_kernel<DR, ROWS><<<grid, WAVE, 0, stream>>>(prep, state, cu_seqlens, seq_slot, raw, H, Hq, d, dv, state_stride)
+  if (wide) {                             // rows a lane: an eighth of the key head, rounded up to the next template
+    if (d <= 32) GD_SCAN(4, 8);
+    else if (d <= 64) GD_SCAN(8, 8);
+    else if (d <= 128) GD_SCAN(16, 8);
+    else GD_SCAN(32, 8);
+  } else {                                // a quarter
+    if (d <= 16) GD_SCAN(4, 4);
+    else if (d <= 32) GD_SCAN(8, 4);
+    else if (d <= 64) GD_SCAN(16, 4);
+    else if (d <= 128) GD_SCAN(32, 4);
+    else GD_SCAN(64, 4);
+  }
 #undef GD_SCAN
   if (int rc = launch_status(); rc != YALM_OK) return rc;
   if (dtype == YALM_F32)
