@@ -37,7 +37,7 @@ __global__ void activate_kernel(const float* __restrict__ z, T* __restrict__ out
 
 // x[t, :] += sigmoid(h[t, :] . w) * y[t, :]; a block a token
 template <typename T, int NW>
-__global__ void gated_add_kernel(const float* __restrict__ y, const T* __restrict__ h, const T* __restrict__ w,
+__global__ __launch_bounds__(NW * WAVE) void gated_add_kernel(const float* __restrict__ y, const T* __restrict__ h, const T* __restrict__ w,
                                  float* __restrict__ x, int D, int accumulate) {
   __shared__ float red[NW];
   const int t = blockIdx.x;
@@ -87,11 +87,16 @@ extern "C" int yalm_gated_add(const float* y, const void* h, const void* w, int 
                               int accumulate, hipStream_t stream) {
   if (T <= 0) return YALM_OK;
   if (D <= 0) return YALM_ERR_ARG;
-  if (dtype == YALM_F32)
-    gated_add_kernel<float, 4><<<T, 256, 0, stream>>>(y, (const float*)h, (const float*)w, x, D, accumulate);
-  else if (dtype == YALM_BF16)
-    gated_add_kernel<bf16, 4><<<T, 256, 0, stream>>>(y, (const bf16*)h, (const bf16*)w, x, D, accumulate);
-  else
+  // a step of few tokens has few workgroups: sixteen waves a token then, four otherwise
+  const bool wide = D >= 2048 && T <= 256;
+  if (dtype == YALM_F32) {
+    if (wide) gated_add_kernel<float, 16><<<T, 1024, 0, stream>>>(y, (const float*)h, (const float*)w, x, D, accumulate);
+    else gated_add_kernel<float, 4><<<T, 256, 0, stream>>>(y, (const float*)h, (const float*)w, x, D, accumulate);
+  } else if (dtype == YALM_BF16) {
+    if (wide) gated_add_kernel<bf16, 16><<<T, 1024, 0, stream>>>(y, (const bf16*)h, (const bf16*)w, x, D, accumulate);
+    else gated_add_kernel<bf16, 4><<<T, 256, 0, stream>>>(y, (const bf16*)h, (const bf16*)w, x, D, accumulate);
+  } else {
     return YALM_ERR_DTYPE;
+  }
   return launch_status();
 }

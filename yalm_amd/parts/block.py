@@ -27,21 +27,35 @@ class PreNormResidualBlock(Part):
         return self.mixer_norm
 
     def forward(self, x, ctx, line, writes_cache=True, next_norm=None):
+        plain_end = False                 # whether the layer's last sublayer ran behind a norm kernel of its own
         if self.mixer.fuses_norm(self.mixer_norm, x, ctx):
             self.mixer.forward_prenorm(x, self.mixer_norm, ctx, line, writes_cache,
                                        emit_for=self.feed_forward_norm if self.feed_forward is not None else next_norm)
         else:
-            h = ctx.ws.get("block.h", (x.shape[0], self.dim), ctx.act_dtype)
-            self.mixer_norm.forward(x, h, ctx)
+            left = ctx.normed.pop(id(self.mixer_norm), None)
+            if left is not None and left[1] is None:      # the layer before has left this norm's output
+                h = left[0]
+            else:
+                h = ctx.ws.get("block.h", (x.shape[0], self.dim), ctx.act_dtype)
+                self.mixer_norm.forward(x, h, ctx)
             self.mixer.forward(h, x, ctx, line, writes_cache)
-        if self.feed_forward is None:
-            return
-        if self.feed_forward.fuses_norm(self.feed_forward_norm, x, ctx):
-            self.feed_forward.forward_prenorm(x, self.feed_forward_norm, ctx, emit_for=next_norm)
-        else:
-            h = ctx.ws.get("block.h", (x.shape[0], self.dim), ctx.act_dtype)
-            self.feed_forward_norm.forward(x, h, ctx)
-            self.feed_forward.forward(h, x, ctx)
+            plain_end = self.feed_forward is None
+        if self.feed_forward is not None:
+            if self.feed_forward.fuses_norm(self.feed_forward_norm, x, ctx):
+                self.feed_forward.forward_prenorm(x, self.feed_forward_norm, ctx, emit_for=next_norm)
+            else:
+                h = ctx.ws.get("block.h", (x.shape[0], self.dim), ctx.act_dtype)
+                self.feed_forward_norm.forward(x, h, ctx)
+                self.feed_forward.forward(h, x, ctx)
+                plain_end = True
+        # sublayers that fold no norm into their products leave nothing for whoever reads the stream next: in a decode
+        # step the layer then ends with that norm as a kernel of its own, so that the head's product (or the next
+        # layer's first) takes its output as it is instead of norming the rows again for every tile of its weights
+        if plain_end and ctx.mode == "decode" and next_norm is not None and hasattr(next_norm, "fused") \
+                and id(next_norm) not in ctx.normed:
+            ahead = ctx.ws.get("block.ahead", (x.shape[0], self.dim), ctx.act_dtype)
+            next_norm.forward(x, ahead, ctx)
+            ctx.normed[id(next_norm)] = (ahead, None, None)
 
 
 @part("block", "parallel_residual")
