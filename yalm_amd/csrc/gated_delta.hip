@@ -15,7 +15,8 @@ namespace {
 
 constexpr int GD_THREADS = 256;
 constexpr int GD_MAX_TAPS = 16;
-constexpr int GD_TOKENS = 16;            // tokens whose operands the scan stages in LDS at a time
+// The scan stages the operands of 16 tokens in LDS at a time, or of 4 in steps of single tokens (a quarter of the LDS and
+// few registers for what waits: more waves a compute unit, whose loads of the state overlap).
 
 __device__ __forceinline__ float sigmoidf_(float z) { return 1.0f / (1.0f + expf(-z)); }
 __device__ __forceinline__ float softplusf_(float z) { return z > 20.f ? z : log1pf(expf(z)); }
@@ -111,7 +112,7 @@ __device__ __forceinline__ float rows_sum(float x) {
   return x;
 }
 
-template <int DR, int GD_ROWS>
+template <int DR, int GD_ROWS, int GD_TOKENS>
 __global__ __launch_bounds__(WAVE) void gd_scan_kernel(const float* __restrict__ prep, float* __restrict__ state,
                                                        const int* __restrict__ cu_seqlens,
                                                        const int* __restrict__ seq_slot, float* __restrict__ raw, int H,
@@ -277,13 +278,19 @@ extern "C" int yalm_gated_delta(const float* proj, const float* low, const float
   const int cols = WAVE / (wide ? 8 : 4);
   if (ceil_div(dv, cols) > 65535) return YALM_ERR_ARG;
   const dim3 grid(ceil_div(dv, cols), H, B);
-#define GD_SCAN(DR, ROWS) \
-  gd_scan_kernel<DR, ROWS><<<grid, WAVE, 0, stream>>>(prep, state, cu_seqlens, seq_slot, raw, H, Hq, d, dv, state_stride)
+  const bool few = T <= 4 * B;
+#define GD_SCAN_(DR, ROWS, TOKENS) \
+  gd_scan_kernel<DR, ROWS, TOKENS><<<grid, WAVE, 0, stream>>>(prep, state, cu_seqlens, seq_slot, raw, H, Hq, d, dv, state_stride)
+#define GD_SCAN(DR, ROWS)             \
+  do {                                \
+    if (few) GD_SCAN_(DR, ROWS, 4);   \
+    else GD_SCAN_(DR, ROWS, 16);      \
+  } while (0)
   if (wide) {                             // rows a lane: an eighth of the key head, rounded up to the next template
-    if (d <= 32) GD_SCAN(4, 8);
-    else if (d <= 64) GD_SCAN(8, 8);
-    else if (d <= 128) GD_SCAN(16, 8);
-    else GD_SCAN(32, 8);
+    if (d <= 32) GD_SCAN_(4, 8, 16);
+    else if (d <= 64) GD_SCAN_(8, 8, 16);
+    else if (d <= 128) GD_SCAN_(16, 8, 16);
+    else GD_SCAN_(32, 8, 16);
   } else {                                // a quarter
     if (d <= 16) GD_SCAN(4, 4);
     else if (d <= 32) GD_SCAN(8, 4);
@@ -292,6 +299,7 @@ extern "C" int yalm_gated_delta(const float* proj, const float* low, const float
     else GD_SCAN(64, 4);
   }
 #undef GD_SCAN
+#undef GD_SCAN_
   if (int rc = launch_status(); rc != YALM_OK) return rc;
   if (dtype == YALM_F32)
     gd_finish_kernel<float><<<dim3(T, H), WAVE, 0, stream>>>(raw, low, w_norm, tok_seq, seq_slot, (float*)out, H, d, dv, eps);
