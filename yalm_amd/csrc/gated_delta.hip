@@ -26,7 +26,7 @@ __device__ __forceinline__ float softplusf_(float z) { return z > 20.f ? z : log
 // prep [T, 2 Kq + Vv + H + H d]: q | k | v | beta | g, ready for the scan.
 // conv_w [2 Kq + Vv, taps], the last column is the current token's.  conv_state [n_slots, state_stride] holds, from
 // conv_off on, [channel][taps - 1] inputs of the tokens before this step, the latest last.
-// grid (T, units): a token's work is cut into units of at most 256 channels so that a step of few tokens still fills
+// grid (T, 1 .. units): a token's work is cut into units of at most 256 channels so that a step of few tokens still fills
 // the chip: unit u < 2 Hq is a query or key head (d <= 256: a thread a channel, the head's sum of squares across the
 // workgroup), the next ceil(Vv / 256) units are the values, the last ceil(H d / 256) the decays (the first of them also
 // the step sizes).
@@ -36,51 +36,59 @@ __global__ __launch_bounds__(GD_THREADS) void gd_prepare_kernel(
     const int* __restrict__ tok_seq, const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slot,
     float* __restrict__ prep, int H, int Hq, int d, int dv, int taps, float q_scale, float unit_floor, long state_stride,
     long conv_off) {
-  __shared__ float part[GD_THREADS / WAVE];
-  const int t = blockIdx.x, unit = blockIdx.y, tid = threadIdx.x;
+  __shared__ float part[2][GD_THREADS / WAVE];
+  const int t = blockIdx.x, tid = threadIdx.x;
   const int Kq = Hq * d, Vv = H * dv, C = 2 * Kq + Vv;
   const int n_in = C + H, n_out = C + H + H * d;
   const int v_units = (Vv + GD_THREADS - 1) / GD_THREADS;
+  const int units = 2 * Hq + v_units + (H * d + GD_THREADS - 1) / GD_THREADS;
   const int b = tok_seq[t];
   const int slot = seq_slot[b];
+  const int p = slot < 0 ? 0 : t - cu_seqlens[b];  // the token's place among its sequence's tokens of this step
   float* out = prep + (size_t)t * n_out;
   const float* x = proj + (size_t)t * n_in;
-  if (unit >= 2 * Hq + v_units) {                 // decays (and step sizes)
-    const int du = unit - 2 * Hq - v_units, i = du * GD_THREADS + tid;
-    if (du == 0)
-      for (int h = tid; h < H; h += GD_THREADS) out[C + h] = slot < 0 ? 0.f : sigmoidf_(x[C + h]);
-    if (i < H * d) {
-      const float z = low[(size_t)t * (H * d + Vv) + i];
-      out[C + H + i] = slot < 0 ? 0.f : expf(-expf(decay_log[i / d]) * softplusf_(z + decay_bias[i]));
+  const float* held = state + (size_t)max(slot, 0) * state_stride + conv_off;
+  // a step of many tokens has workgroups enough: each then walks several units (gridDim.y apart, so heads come before
+  // values before decays in every workgroup) and has found its token's sequence once
+  for (int unit = blockIdx.y, round = 0; unit < units; unit += gridDim.y, ++round) {
+    if (unit >= 2 * Hq + v_units) {               // decays (and step sizes)
+      const int du = unit - 2 * Hq - v_units, i = du * GD_THREADS + tid;
+      if (du == 0)
+        for (int h = tid; h < H; h += GD_THREADS) out[C + h] = slot < 0 ? 0.f : sigmoidf_(x[C + h]);
+      if (i < H * d) {
+        const float z = low[(size_t)t * (H * d + Vv) + i];
+        out[C + H + i] = slot < 0 ? 0.f : expf(-expf(decay_log[i / d]) * softplusf_(z + decay_bias[i]));
+      }
+      continue;
     }
-    return;
-  }
-  const bool head = unit < 2 * Hq;
-  const int c = head ? unit * d + tid : 2 * Kq + (unit - 2 * Hq) * GD_THREADS + tid;
-  const bool live = head ? tid < d : c < C;
-  float a = 0.f;
-  if (live && slot >= 0) {
-    const int p = t - cu_seqlens[b];              // the token's place among its sequence's tokens of this step
-    const float* held = state + (size_t)slot * state_stride + conv_off;
-    const float* w = conv_w + (size_t)c * taps;
-    float acc = w[taps - 1] * x[c];
-    for (int back = 1; back < taps; ++back) {
-      const float past = back <= p ? proj[(size_t)(t - back) * n_in + c] : held[(size_t)c * (taps - 1) + (taps - 1 - back + p)];
-      acc = fmaf(w[taps - 1 - back], past, acc);
+    const bool head = unit < 2 * Hq;
+    const int c = head ? unit * d + tid : 2 * Kq + (unit - 2 * Hq) * GD_THREADS + tid;
+    const bool live = head ? tid < d : c < C;
+    float a = 0.f;
+    if (live && slot >= 0) {
+      const float* w = conv_w + (size_t)c * taps;
+      float acc = w[taps - 1] * x[c];
+      for (int back = 1; back < taps; ++back) {
+        const float past = back <= p ? proj[(size_t)(t - back) * n_in + c] : held[(size_t)c * (taps - 1) + (taps - 1 - back + p)];
+        acc = fmaf(w[taps - 1 - back], past, acc);
+      }
+      a = acc / (1.0f + expf(-acc));
     }
-    a = acc / (1.0f + expf(-acc));
-  }
-  if (!head) {
-    if (live) out[c] = a;
-    return;
-  }
-  const float ss = wave_sum(a * a);               // unit vectors: the head's sum of squares across the workgroup
-  if (tid % WAVE == 0) part[tid / WAVE] = ss;
-  __syncthreads();
-  float total = 0.f;
+    if (!head) {
+      if (live) out[c] = a;
+      continue;
+    }
+    // unit vectors: the head's sum of squares across the workgroup (the rounds alternate between two sets of partial
+    // sums, and a round's barrier stands between the reads of a set and its next writes)
+    float* mine = part[round & 1];
+    const float ss = wave_sum(a * a);
+    if (tid % WAVE == 0) mine[tid / WAVE] = ss;
+    __syncthreads();
+    float total = 0.f;
 #pragma unroll
-  for (int w = 0; w < GD_THREADS / WAVE; ++w) total += part[w];
-  if (live) out[c] = slot < 0 ? 0.f : a * ((unit < Hq ? q_scale : 1.0f) / sqrtf(total + unit_floor));
+    for (int w = 0; w < GD_THREADS / WAVE; ++w) total += mine[w];
+    if (live) out[c] = slot < 0 ? 0.f : a * ((unit < Hq ? q_scale : 1.0f) / sqrtf(total + unit_floor));
+  }
 }
 
 // The convolutions' inputs that the next step needs: the last taps - 1 of (what was held) ++ (this step's).
@@ -180,19 +188,27 @@ __global__ __launch_bounds__(WAVE) void gd_scan_kernel(const float* __restrict__
     if (lane < GD_TOKENS) sb[lane] = pb;
     __syncthreads();
     if (c0 + GD_TOKENS < t1) fetch(c0 + GD_TOKENS);
-#pragma unroll 2
-    for (int tt = 0; tt < n; ++tt) {
-      // the token's operands for this lane's rows, four at a time (a row group starts on a 16-byte border)
+    // A token's operands for this lane's rows come from LDS four at a time (a row group starts on a 16-byte border),
+    // and the NEXT token's are asked for before the token at hand is worked: two sets of registers take turns.
+    struct Ops {
+      float4 g[DR / 4], k[DR / 4], q[DR / 4];
+      float beta, v;
+    };
+    auto take = [&](Ops& o, int tt) {
       const float4* g4 = reinterpret_cast<const float4*>(&sg[tt][r * LD]);
       const float4* k4 = reinterpret_cast<const float4*>(&sk[tt][r * LD]);
       const float4* q4 = reinterpret_cast<const float4*>(&sq[tt][r * LD]);
-      float kk[DR];
+#pragma unroll
+      for (int v = 0; v < DR / 4; ++v) o.g[v] = g4[v], o.k[v] = k4[v], o.q[v] = q4[v];
+      o.beta = sb[tt];
+      o.v = sv[tt][c];
+    };
+    auto work = [&](const Ops& o, int tt) {
       float kv0 = 0.f, kv1 = 0.f, kv2 = 0.f, kv3 = 0.f;
 #pragma unroll
       for (int v = 0; v < DR / 4; ++v) {
-        const float4 g = g4[v], k = k4[v];
+        const float4 g = o.g[v], k = o.k[v];
         const int i = 4 * v;
-        kk[i] = k.x, kk[i + 1] = k.y, kk[i + 2] = k.z, kk[i + 3] = k.w;
         S[i] *= g.x, S[i + 1] *= g.y, S[i + 2] *= g.z, S[i + 3] *= g.w;
         kv0 = fmaf(S[i], k.x, kv0);
         kv1 = fmaf(S[i + 1], k.y, kv1);
@@ -200,23 +216,41 @@ __global__ __launch_bounds__(WAVE) void gd_scan_kernel(const float* __restrict__
         kv3 = fmaf(S[i + 3], k.w, kv3);
       }
       const float kv = rows_sum<GD_ROWS>((kv0 + kv1) + (kv2 + kv3));
-      const float u = sb[tt] * (sv[tt][c] - kv);
+      const float u = o.beta * (o.v - kv);
       float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
 #pragma unroll
       for (int v = 0; v < DR / 4; ++v) {
-        const float4 q = q4[v];
+        const float4 k = o.k[v], q = o.q[v];
         const int i = 4 * v;
-        S[i] = fmaf(kk[i], u, S[i]);
-        S[i + 1] = fmaf(kk[i + 1], u, S[i + 1]);
-        S[i + 2] = fmaf(kk[i + 2], u, S[i + 2]);
-        S[i + 3] = fmaf(kk[i + 3], u, S[i + 3]);
+        S[i] = fmaf(k.x, u, S[i]);
+        S[i + 1] = fmaf(k.y, u, S[i + 1]);
+        S[i + 2] = fmaf(k.z, u, S[i + 2]);
+        S[i + 3] = fmaf(k.w, u, S[i + 3]);
         o0 = fmaf(S[i], q.x, o0);
         o1 = fmaf(S[i + 1], q.y, o1);
         o2 = fmaf(S[i + 2], q.z, o2);
         o3 = fmaf(S[i + 3], q.w, o3);
       }
-      const float o = rows_sum<GD_ROWS>((o0 + o1) + (o2 + o3));
-      if (live && r == 0) raw[(size_t)(c0 + tt) * Vv + h * dv + j] = o;
+      const float res = rows_sum<GD_ROWS>((o0 + o1) + (o2 + o3));
+      if (live && r == 0) raw[(size_t)(c0 + tt) * Vv + h * dv + j] = res;
+    };
+    Ops A;
+    if constexpr (GD_TOKENS <= 4) {                // steps of single tokens: nothing to ask for ahead
+      for (int tt = 0; tt < n; ++tt) {
+        take(A, tt);
+        work(A, tt);
+      }
+    } else {
+      Ops B;
+      take(A, 0);
+      for (int tt = 0; tt < n; tt += 2) {
+        take(B, min(tt + 1, GD_TOKENS - 1));       // rows behind the step's last token hold zeros or older operands: unused
+        work(A, tt);
+        if (tt + 1 < n) {
+          take(A, min(tt + 2, GD_TOKENS - 1));
+          work(B, tt + 1);
+        }
+      }
     }
   }
   if (live) {
@@ -264,7 +298,9 @@ extern "C" int yalm_gated_delta(const float* proj, const float* low, const float
   const long conv_off = (long)H * d * dv, state_stride = conv_off + (long)C * (taps - 1);
   const int units = 2 * Hq + ceil_div(H * dv, GD_THREADS) + ceil_div(H * d, GD_THREADS);
   if (units > 65535 || d > GD_THREADS) return YALM_ERR_ARG;
-  gd_prepare_kernel<<<dim3(T, units), GD_THREADS, 0, stream>>>(proj, low, conv_w, decay_log, decay_bias, state, tok_seq, cu_seqlens,
+  // about 16 thousand workgroups at least, none with more units than there are
+  const int unit_rows = min(units, max(1, ceil_div(16384, T)));
+  gd_prepare_kernel<<<dim3(T, unit_rows), GD_THREADS, 0, stream>>>(proj, low, conv_w, decay_log, decay_bias, state, tok_seq, cu_seqlens,
                                                     seq_slot, prep, H, Hq, d, dv, taps, q_scale, unit_floor, state_stride,
                                                     conv_off);
   if (int rc = launch_status(); rc != YALM_OK) return rc;
@@ -287,10 +323,10 @@ extern "C" int yalm_gated_delta(const float* proj, const float* low, const float
     else GD_SCAN_(DR, ROWS, 16);      \
   } while (0)
   if (wide) {                             // rows a lane: an eighth of the key head, rounded up to the next template
-    if (d <= 32) GD_SCAN_(4, 8, 16);
-    else if (d <= 64) GD_SCAN_(8, 8, 16);
-    else if (d <= 128) GD_SCAN_(16, 8, 16);
-    else GD_SCAN_(32, 8, 16);
+    if (d <= 32) GD_SCAN_(4, 8, 16);          // eight tokens' operands at a time where a lane has many rows: fewer
+    else if (d <= 64) GD_SCAN_(8, 8, 16);     // registers wait with the next tokens' operands
+    else if (d <= 128) GD_SCAN_(16, 8, 8);
+    else GD_SCAN_(32, 8, 8);
   } else {                                // a quarter
     if (d <= 16) GD_SCAN(4, 4);
     else if (d <= 32) GD_SCAN(8, 4);
