@@ -113,6 +113,9 @@ def _load(a):
         with open(a["random"]) as f:
             cfg = config_from_dict(json.load(f))
         if a["context"]:
+            if not hasattr(cfg, "with_context"):
+                sys.stderr.write("Error: -T is not offered for the %s design\n" % getattr(cfg, "architecture", type(cfg).__name__))
+                raise SystemExit(1)
             cfg = cfg.with_context(a["context"])
         return Model.random(cfg, a["weight_seed"], dtype=dtype, device="cuda:0")
     model = Model.from_folder(a["checkpoint"], dtype=dtype, device="cuda:0", context=a["context"])

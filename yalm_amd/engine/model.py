@@ -87,10 +87,12 @@ class Model:
         the last `window` positions only; context: the reference's -T (attention sinks and a window
         that fill a context of that many positions)."""
         cfg = config_from_folder(path)
-        if window:
-            cfg = cfg.with_window(window)
-        if context:
-            cfg = cfg.with_context(context)
+        for value, how in ((window, "with_window"), (context, "with_context")):
+            if value:
+                if not hasattr(cfg, how):     # a design whose layers say themselves what each attention sees
+                    raise ValueError("a window or context from outside is not offered for the %s design"
+                                     % getattr(cfg, "architecture", type(cfg).__name__))
+                cfg = getattr(cfg, how)(value)
         model = cls(cfg.to_spec(), cfg)
         source = TensorSource(path)
         source.check(model.param_specs(), strict=strict)
