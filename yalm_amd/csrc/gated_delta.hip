@@ -5,7 +5,7 @@
 //   S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q          (the read-out sees the token's own write)
 // Every column of S runs this on its own, so four lanes own one column, held in registers, and walk the tokens in order.
 //
-// Three kernels a step: `prepare` turns a token's projections into the recurrence's operands (the short causal
+// Four kernels a step: `prepare` turns a token's projections into the recurrence's operands (the short causal
 // convolutions with silu, the unit vectors, sigmoid and the decays), `carry` moves the convolutions' last inputs into
 // the per-sequence state, `scan` runs the recurrence and `finish` norms the heads' results and gates them.
 #include "common.h"
