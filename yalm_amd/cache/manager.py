@@ -52,6 +52,11 @@ class StateRequest:
     dtype: torch.dtype = torch.float32
 
 
+def _line_order(line):
+    """Storage order of cache lines: the plain numbers first, then the lines of a layer's members, (number, name)."""
+    return (0, line, "") if isinstance(line, int) else (1, 0, repr(line))
+
+
 def pages_for(n_tokens):
     return (n_tokens + PAGE - 1) // PAGE
 
@@ -246,7 +251,8 @@ class StateGroup:
 class CacheManager:
     """Slots, pages and state for all cache lines of a model.
 
-    requests: {cache line id: KVRequest | StateRequest | None}
+    requests: {cache line id: KVRequest | StateRequest | None, or {name: such a request, or such a dictionary}: a
+    layer made of several members that keep something has the line (id, name) for each}
     max_tokens: the most tokens live sequences hold at any time, each sequence's
     count rounded up to a multiple of PAGE."""
 
@@ -261,18 +267,24 @@ class CacheManager:
         self.slots = SlotAllocator(self.n_slots)
         self.seq_len = [0] * self.n_slots
         by_request = {}
-        for line, req in requests.items():
-            if req is not None:
+
+        def enter(line, req):
+            if isinstance(req, dict):
+                for name, sub in req.items():
+                    enter((line, name), sub)
+            elif req is not None:
                 by_request.setdefault(req, []).append(line)
+        for line, req in requests.items():
+            enter(line, req)
         self.kv_groups = []
         self.state_groups = []
         self._group_of_line = {}
         for req, lines in by_request.items():
             if isinstance(req, KVRequest):
-                g = KVGroup(req, sorted(lines), self.n_pages, self.n_slots, self.max_seq_len, dtype, device)
+                g = KVGroup(req, sorted(lines, key=_line_order), self.n_pages, self.n_slots, self.max_seq_len, dtype, device)
                 self.kv_groups.append(g)
             elif isinstance(req, StateRequest):
-                g = StateGroup(req, sorted(lines), self.n_slots, device)
+                g = StateGroup(req, sorted(lines, key=_line_order), self.n_slots, device)
                 self.state_groups.append(g)
             else:
                 raise CacheError("unknown cache request %r" % (req,))

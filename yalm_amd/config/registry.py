@@ -9,6 +9,7 @@ import os
 from .llama import ConfigError, LlamaConfig
 from .bovozen import BovozenConfig
 from .gedunex import GedunexConfig
+from .rekirax import RekiraxConfig
 from .situlorn import SitulornConfig
 
 _ARCHITECTURES = {}
@@ -63,6 +64,6 @@ def _folder_shapes(path):
     return shapes.get
 
 
-for _cls in (LlamaConfig, SitulornConfig, GedunexConfig, BovozenConfig):
+for _cls in (LlamaConfig, SitulornConfig, GedunexConfig, BovozenConfig, RekiraxConfig):
     for _name in _cls.ARCHITECTURES:
         register_architecture(_name, _cls)

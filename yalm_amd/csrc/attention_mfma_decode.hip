@@ -85,6 +85,8 @@ __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_k
 
     const float* bias_row = BIAS && bias != nullptr ? bias + (size_t)(h0 + min(j, G - 1)) * n_bias : nullptr;   // the column's head
     const float slope2 = BIAS && shape.slope != nullptr ? shape.slope[h0 + min(j, G - 1)] * 1.4426950408889634f : 0.f;
+    const bool log_term = BIAS && shape.log_a != nullptr;
+    const float log_a = log_term ? shape.log_a[h0 + min(j, G - 1)] : 0.f, log_b = log_term ? shape.log_b[h0 + min(j, G - 1)] : 0.f;
     bf16x8 kreg[4][KS];
     auto page_of = [&](int a) { return min(max(table[a % ring_pages], 0), n_pages - 1); };
     auto load_keys = [&](int phys) {
@@ -142,6 +144,7 @@ __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_k
               v = soft_cap_fast(v * LN2, shape.softcap) * 1.4426950408889634f;
             if (bias_row != nullptr) v = fmaf(bias_row[min(max(dist, 0), n_bias - 1)], 1.4426950408889634f, v);
             v = fmaf(-slope2, (float)dist, v);
+            if (log_term) v += log_distance_term2(log_a, log_b, dist);
           }
           if (edge) {
             int pos = base + 32 * (t >> 1) + 8 * qd + 4 * (t & 1) + r;

@@ -75,6 +75,8 @@ __global__ __launch_bounds__(256 * KSPL, KSPL == 1 ? 2 : 1) void attn_prefill_mf
   const float score_scale = 1.4426950408889634f / sqrtf((float)HD);   // log2(e) / sqrt(head_dim)
   const float* bias_row = BIAS && bias != nullptr ? bias + (size_t)h * n_bias : nullptr;
   const float slope2 = BIAS && shape.slope != nullptr ? shape.slope[h] * 1.4426950408889634f : 0.f;   // in exponents of 2
+  const bool log_term = BIAS && shape.log_a != nullptr;
+  const float log_a = log_term ? shape.log_a[h] : 0.f, log_b = log_term ? shape.log_b[h] : 0.f;
 
   const int blk0 = tq * PAGE;                     // first position of the workgroup
   const int pos0 = blk0 + wave * 16 * NC;         // first position of the wave
@@ -190,6 +192,7 @@ __global__ __launch_bounds__(256 * KSPL, KSPL == 1 ? 2 : 1) void attn_prefill_mf
                 const int dist = pos_q[c] - (base + 32 * (t >> 1) + 8 * qd + 4 * (t & 1) + r);
                 float term = bias_row != nullptr ? bias_row[min(max(dist, 0), n_bias - 1)] * 1.4426950408889634f : 0.f;
                 term = fmaf(-slope2, (float)dist, term);
+                if (log_term) term += log_distance_term2(log_a, log_b, dist);
                 if (shape.softcap > 0.f)           // capped in natural units, then into exponents of 2
                   v = fmaf(soft_cap_fast(v * (score_scale * LN2), shape.softcap), 1.4426950408889634f, term);
                 else

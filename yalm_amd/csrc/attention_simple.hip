@@ -30,9 +30,12 @@ struct ScoreBias {
   const float* sink_logit;     // [heads]: one more term exp(sink_logit[head]) of the softmax's denominator, without a key (null: none)
   const float* slope;          // [heads]: -slope[head] * distance is added to every score (null: none)
   int block;                   // a query sees the keys of its own block of `block` positions only (0: no blocks)
+  const float* log_a;          // [heads], with log_b [heads]: -log_a[head] ln(1 + log_b[head] distance) is added (null: none)
+  const float* log_b;
   __device__ __forceinline__ float at(int head, int distance) const {
     float term = table != nullptr ? table[(size_t)head * n + min(max(distance, 0), n - 1)] : 0.f;
     if (slope != nullptr) term -= slope[head] * (float)distance;
+    if (log_a != nullptr) term -= log_a[head] * log1pf(log_b[head] * (float)max(distance, 0));
     return term;
   }
   // the score of a scaled product at a distance
@@ -338,12 +341,13 @@ extern "C" int yalm_attn_prefill_lse(const void* q, const void* k_stage, const v
                                  const int* tile_order, int n_order, int T, int B, int n_tiles, int n_heads,
                                  int n_kv_heads, int head_dim, int window, int dtype, int force_simple,
                                  const float* score_bias, int n_bias, float softcap, const float* sink_logit,
-                                 const float* slopes, int block, hipStream_t stream) {
+                                 const float* slopes, int block, const float* log_a, const float* log_b,
+                                 hipStream_t stream) {
   if (T <= 0) return YALM_OK;
   if (bad_heads(n_heads, n_kv_heads, head_dim) || window < 0 || block < 0 || n_tiles <= 0) return YALM_ERR_ARG;
   if ((score_bias != nullptr && n_bias <= 0) || softcap < 0.f) return YALM_ERR_ARG;
-  const ScoreBias sb = {score_bias, n_bias, softcap, sink_logit, slopes, block};
-  const ScoreShape shape = {score_bias, n_bias, softcap, sink_logit, slopes, block};
+  const ScoreBias sb = {score_bias, n_bias, softcap, sink_logit, slopes, block, log_a, log_b};
+  const ScoreShape shape = {score_bias, n_bias, softcap, sink_logit, slopes, block, log_a, log_b};
   dim3 grid(T, n_heads);
   if (dtype == YALM_F32) {
     if (head_dim <= ACC_SMALL * WAVE)
@@ -380,7 +384,7 @@ extern "C" int yalm_attn_prefill(const void* q, const void* k_stage, const void*
                                  hipStream_t stream) {
   return yalm_attn_prefill_lse(q, k_stage, v_stage, out, nullptr, nullptr, cu_seqlens, seq_tile0, tok_seq, tok_pos, tile_order,
                                n_order, T, B, n_tiles, n_heads, n_kv_heads, head_dim, window, dtype, force_simple,
-                               nullptr, 0, 0.f, nullptr, nullptr, 0, stream);
+                               nullptr, 0, 0.f, nullptr, nullptr, 0, nullptr, nullptr, stream);
 }
 
 // merges the partial results of the splits (also used by the MFMA kernel)
@@ -407,12 +411,13 @@ int attn_decode_any(const void* q, const void* k_pages, const void* v_pages, con
                     int B, int n_heads, int n_kv_heads, int head_dim, int window, int n_splits, int n_pages,
                     int page_layout, int dtype, int force_simple, const SinkArgs& sinks, const int* step_max_len,
                     const int* seq_order, const float* score_bias, int n_bias, float softcap,
-                    const float* sink_logit, const float* slopes, int block, hipStream_t stream) {
+                    const float* sink_logit, const float* slopes, int block, const float* log_a, const float* log_b,
+                                 hipStream_t stream) {
   if (B <= 0) return YALM_OK;
-  const ScoreShape shape = {score_bias, n_bias, softcap, sink_logit, slopes, block};
+  const ScoreShape shape = {score_bias, n_bias, softcap, sink_logit, slopes, block, log_a, log_b};
   if ((score_bias != nullptr && n_bias <= 0) || softcap < 0.f || block < 0 || ((shape.any() || block > 0) && sinks.n_sinks > 0))
     return YALM_ERR_ARG;                                                // kept first positions are scored unshaped
-  const ScoreBias sb = {score_bias, n_bias, softcap, sink_logit, slopes, block};
+  const ScoreBias sb = {score_bias, n_bias, softcap, sink_logit, slopes, block, log_a, log_b};
   if (bad_heads(n_heads, n_kv_heads, head_dim) || window < 0 || n_splits <= 0 || ring_pages <= 0 ||
       !page_layout_ok(page_layout, head_dim))
     return YALM_ERR_ARG;
@@ -463,11 +468,13 @@ extern "C" int yalm_attn_decode_lse(const void* q, const void* k_pages, const vo
                                     int head_dim, int window, int n_splits, int n_pages, int page_layout, int dtype,
                                     int force_simple, const int* step_max_len, const int* seq_order,
                                     const float* score_bias, int n_bias, float softcap, const float* sink_logit,
-                                    const float* slopes, int block, hipStream_t stream) {
+                                    const float* slopes, int block, const float* log_a, const float* log_b,
+                                 hipStream_t stream) {
   SinkArgs none = {};
   return attn_decode_any(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len, out, lse,
                          partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout, dtype,
-                         force_simple, none, step_max_len, seq_order, score_bias, n_bias, softcap, sink_logit, slopes, block, stream);
+                         force_simple, none, step_max_len, seq_order, score_bias, n_bias, softcap, sink_logit, slopes, block,
+                         log_a, log_b, stream);
 }
 
 extern "C" int yalm_attn_decode(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
@@ -476,7 +483,7 @@ extern "C" int yalm_attn_decode(const void* q, const void* k_pages, const void* 
                                 int n_splits, int n_pages, int dtype, int force_simple, hipStream_t stream) {
   return yalm_attn_decode_lse(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len, out,
                               nullptr, partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages,
-                              YALM_PAGE_ROWS, dtype, force_simple, nullptr, nullptr, nullptr, 0, 0.f, nullptr, nullptr, 0, stream);
+                              YALM_PAGE_ROWS, dtype, force_simple, nullptr, nullptr, nullptr, 0, 0.f, nullptr, nullptr, 0, nullptr, nullptr, stream);
 }
 
 extern "C" int yalm_attn_decode_sinks(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
@@ -512,7 +519,7 @@ extern "C" int yalm_attn_decode_sinks(const void* q, const void* k_pages, const 
   sk.n_sinks = n_sinks;
   return attn_decode_any(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len, out, nullptr,
                          partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout, dtype,
-                         force_simple, sk, step_max_len, seq_order, nullptr, 0, 0.f, nullptr, nullptr, 0, stream);
+                         force_simple, sk, step_max_len, seq_order, nullptr, 0, 0.f, nullptr, nullptr, 0, nullptr, nullptr, stream);
 }
 
 // ---------------------------------------------------------------------------

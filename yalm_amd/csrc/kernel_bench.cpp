@@ -134,7 +134,7 @@ int main(int argc, char** argv) {
       for (int c = 0; c < launches; ++c) {
         int rc = yalm_attn_decode_lse(q, kp, vp, (const int*)d_table, pages_seq, pages_seq, (const int*)d_slot,
                                       (const int*)d_len, out, nullptr, partial, B, n_heads, n_kv, hd, 0, n_splits,
-                                      B * pages_seq, /* pages in blocks */ 1, /* bfloat16 */ 1, 0, nullptr, nullptr, nullptr, 0, 0.f, nullptr, nullptr, 0, stream);
+                                      B * pages_seq, /* pages in blocks */ 1, /* bfloat16 */ 1, 0, nullptr, nullptr, nullptr, 0, 0.f, nullptr, nullptr, 0, nullptr, nullptr, stream);
         if (rc != 0) {
           fprintf(stderr, "yalm_attn_decode_lse failed: %s\n", yalm_error_string(rc));
           return 1;

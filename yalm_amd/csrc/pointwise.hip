@@ -1,5 +1,7 @@
 // Small per-row kernels: an embedding with a learned position vector, an activation between the two products of an
-// ungated feed-forward, and the add of a sublayer's result under a gate of one number a token.
+// ungated feed-forward (or of a gated one whose products carry biases), the add of a sublayer's result under a gate
+// of one number a token, a short causal convolution over time on every channel with its carried inputs, a sigmoid
+// gate on an attention's heads, and the way into a walk of looped layers.
 #include "common.h"
 #include "yalm_hip.h"
 
@@ -51,6 +53,100 @@ __global__ __launch_bounds__(NW * WAVE) void gated_add_kernel(const float* __res
   for (int i = threadIdx.x; i < D; i += NW * WAVE) xr[i] = accumulate ? fmaf(s, yr[i], xr[i]) : s * yr[i];
 }
 
+// out[t, c] = (residual ? h[t, c] : 0) + sum_j w[c, j] in(t - (taps - 1) + j, c): a causal convolution over the tokens
+// of a sequence, the last tap on the token itself.  Inputs in front of the step's first token of a sequence come from
+// carried[slot][taps - 1][D] (the sequence's last taps - 1 inputs, the newest last; zeros for a new sequence), and a
+// padding row (slot -1) reads zeros there.  A thread a (token, channel).
+template <typename T, int MAX_TAPS>
+__global__ void time_conv_kernel(const T* __restrict__ h, const float* __restrict__ w, const float* __restrict__ carried,
+                                 T* __restrict__ out, const int* __restrict__ tok_seq, const int* __restrict__ cu_seqlens,
+                                 const int* __restrict__ seq_slot, int D, int taps, int residual) {
+  const int t = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= D) return;
+  const int b = tok_seq[t];
+  const int first = b >= 0 ? cu_seqlens[b] : t, slot = b >= 0 ? seq_slot[b] : -1;
+  const int l = t - first;                        // the token's place among its sequence's tokens of this step
+  float acc = residual ? to_f32(h[(size_t)t * D + c]) : 0.f;
+  for (int j = 0; j < taps; ++j) {
+    const int src = l - (taps - 1) + j;
+    float v = 0.f;
+    if (src >= 0) v = to_f32(h[(size_t)(first + src) * D + c]);
+    else if (slot >= 0) v = carried[((size_t)slot * (taps - 1) + (taps - 1 + src)) * D + c];
+    acc = fmaf(w[(size_t)c * taps + j], v, acc);
+  }
+  out[(size_t)t * D + c] = from_f32<T>(acc);
+}
+
+// carried[slot] <- the last taps - 1 inputs of each sequence after this step's tokens; a thread a (sequence, channel)
+// reads what it needs of the old rows before it writes the new ones
+template <typename T, int MAX_TAPS>
+__global__ void time_conv_carry_kernel(const T* __restrict__ h, float* __restrict__ carried,
+                                       const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slot, int D,
+                                       int taps) {
+  const int b = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= D) return;
+  const int slot = seq_slot[b];
+  if (slot < 0) return;
+  const int first = cu_seqlens[b], n = cu_seqlens[b + 1] - first, keep = taps - 1;
+  float* rows = carried + (size_t)slot * keep * D + c;
+  float fresh[MAX_TAPS];
+#pragma unroll
+  for (int i = 0; i < MAX_TAPS; ++i) {
+    if (i < keep) {
+      const int src = n - keep + i;               // place among this step's tokens; negative: an older input
+      fresh[i] = src >= 0 ? to_f32(h[(size_t)(first + src) * D + c]) : rows[(size_t)(keep + src) * D];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < MAX_TAPS; ++i)
+    if (i < keep) rows[(size_t)i * D] = fresh[i];
+}
+
+// out[t, i] = act(z[t, i] + bias[i]) * (z[t, F + i] + bias[F + i]) for i < F: the middle of a gated feed-forward whose
+// two first products (gate | up, float32) carry biases; x[t, :] += x_bias (the second product's bias, which that
+// product's adding epilogue does not know) on the way.  A workgroup a token.
+template <typename T>
+__global__ void gated_bias_act_kernel(const float* __restrict__ z, const float* __restrict__ bias, T* __restrict__ out,
+                                      int F, int kind, float* __restrict__ x, const float* __restrict__ x_bias, int D) {
+  const int t = blockIdx.x;
+  const float* zr = z + (size_t)t * 2 * F;
+  for (int i = threadIdx.x; i < F; i += blockDim.x) {
+    const float v = zr[i] + (bias != nullptr ? bias[i] : 0.f), u = zr[F + i] + (bias != nullptr ? bias[F + i] : 0.f);
+    float a;
+    if (kind == 0) a = 0.5f * v * (1.0f + erff(v * 0.7071067811865476f));
+    else if (kind == 1) a = 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
+    else a = v / (1.0f + expf(-v));
+    out[(size_t)t * F + i] = from_f32<T>(a * u);
+  }
+  if (x_bias != nullptr)
+    for (int i = threadIdx.x; i < D; i += blockDim.x) x[(size_t)t * D + i] += x_bias[i];
+}
+
+// o[t, h, e] *= sigmoid(g[t * g_stride + h * dv + e]) for e < dv (heads of o are `pad` wide); a workgroup a token
+template <typename T>
+__global__ void sigmoid_gate_kernel(T* __restrict__ o, const float* __restrict__ g, long g_stride, int n_heads, int dv,
+                                    int pad) {
+  const int t = blockIdx.x;
+  for (int i = threadIdx.x; i < n_heads * dv; i += blockDim.x) {
+    const int h = i / dv, e = i - h * dv;
+    T* p = o + ((size_t)t * n_heads + h) * pad + e;
+    *p = from_f32<T>(to_f32(*p) / (1.0f + expf(-g[(size_t)t * g_stride + i])));
+  }
+}
+
+// both[t] = [x[t] | x0[t]] in the compute dtype, then x[t] = start: what the product that enters a walk of looped
+// layers reads, and what its adding epilogue adds to
+template <typename T>
+__global__ void loop_pack_kernel(float* __restrict__ x, const float* __restrict__ x0, const float* __restrict__ start,
+                                 T* __restrict__ both, int D) {
+  const int t = blockIdx.x;
+  for (int i = threadIdx.x; i < D; i += blockDim.x) {
+    both[(size_t)t * 2 * D + i] = from_f32<T>(x[(size_t)t * D + i]);
+    both[(size_t)t * 2 * D + D + i] = from_f32<T>(x0[(size_t)t * D + i]);
+    x[(size_t)t * D + i] = start[i];
+  }
+}
+
 }  // namespace
 
 extern "C" int yalm_embed_learned(const void* table, const void* pos_table, int dtype, const int* tokens,
@@ -98,5 +194,73 @@ extern "C" int yalm_gated_add(const float* y, const void* h, const void* w, int 
   } else {
     return YALM_ERR_DTYPE;
   }
+  return launch_status();
+}
+
+constexpr int CONV_MAX_TAPS = 16;
+extern "C" int yalm_time_conv(const void* h, const float* w, float* carried, void* out, const int* tok_seq,
+                              const int* cu_seqlens, const int* seq_slot, int T, int B, int D, int taps, int residual,
+                              int dtype, hipStream_t stream) {
+  if (T <= 0) return YALM_OK;
+  if (D <= 0 || B <= 0 || taps <= 0 || taps > CONV_MAX_TAPS || h == out ||
+      (taps > 1 && carried == nullptr) || ceil_div(D, 256) > 65535)
+    return YALM_ERR_ARG;
+  const int threads = D >= 256 ? 256 : 64;
+  dim3 grid(T, ceil_div(D, threads)), cgrid(B, ceil_div(D, threads));
+  if (dtype == YALM_F32) {
+    time_conv_kernel<float, CONV_MAX_TAPS><<<grid, threads, 0, stream>>>((const float*)h, w, carried, (float*)out, tok_seq,
+                                                                         cu_seqlens, seq_slot, D, taps, residual);
+    if (taps > 1)
+      time_conv_carry_kernel<float, CONV_MAX_TAPS><<<cgrid, threads, 0, stream>>>((const float*)h, carried, cu_seqlens, seq_slot, D, taps);
+  } else if (dtype == YALM_BF16) {
+    time_conv_kernel<bf16, CONV_MAX_TAPS><<<grid, threads, 0, stream>>>((const bf16*)h, w, carried, (bf16*)out, tok_seq,
+                                                                        cu_seqlens, seq_slot, D, taps, residual);
+    if (taps > 1)
+      time_conv_carry_kernel<bf16, CONV_MAX_TAPS><<<cgrid, threads, 0, stream>>>((const bf16*)h, carried, cu_seqlens, seq_slot, D, taps);
+  } else {
+    return YALM_ERR_DTYPE;
+  }
+  return launch_status();
+}
+
+extern "C" int yalm_gated_bias_act(const float* z, const float* bias, void* out, int T, int F, int kind, int out_dtype,
+                                   float* x, const float* x_bias, int D, hipStream_t stream) {
+  if (T <= 0) return YALM_OK;
+  if (F <= 0 || kind < 0 || kind > 2 || (x_bias != nullptr && (x == nullptr || D <= 0))) return YALM_ERR_ARG;
+  const int threads = F >= 2048 ? 1024 : 256;
+  if (out_dtype == YALM_F32)
+    gated_bias_act_kernel<float><<<T, threads, 0, stream>>>(z, bias, (float*)out, F, kind, x, x_bias, D);
+  else if (out_dtype == YALM_BF16)
+    gated_bias_act_kernel<bf16><<<T, threads, 0, stream>>>(z, bias, (bf16*)out, F, kind, x, x_bias, D);
+  else
+    return YALM_ERR_DTYPE;
+  return launch_status();
+}
+
+extern "C" int yalm_sigmoid_gate(void* o, const float* g, long g_stride, int T, int n_heads, int dv, int pad, int dtype,
+                                 hipStream_t stream) {
+  if (T <= 0) return YALM_OK;
+  if (n_heads <= 0 || dv <= 0 || pad < dv || g_stride < (long)n_heads * dv) return YALM_ERR_ARG;
+  const int threads = n_heads * dv >= 2048 ? 1024 : 256;
+  if (dtype == YALM_F32)
+    sigmoid_gate_kernel<float><<<T, threads, 0, stream>>>((float*)o, g, g_stride, n_heads, dv, pad);
+  else if (dtype == YALM_BF16)
+    sigmoid_gate_kernel<bf16><<<T, threads, 0, stream>>>((bf16*)o, g, g_stride, n_heads, dv, pad);
+  else
+    return YALM_ERR_DTYPE;
+  return launch_status();
+}
+
+extern "C" int yalm_loop_pack(float* x, const float* x0, const float* start, void* both, int T, int D, int dtype,
+                              hipStream_t stream) {
+  if (T <= 0) return YALM_OK;
+  if (D <= 0) return YALM_ERR_ARG;
+  const int threads = D >= 2048 ? 1024 : 256;
+  if (dtype == YALM_F32)
+    loop_pack_kernel<float><<<T, threads, 0, stream>>>(x, x0, start, (float*)both, D);
+  else if (dtype == YALM_BF16)
+    loop_pack_kernel<bf16><<<T, threads, 0, stream>>>(x, x0, start, (bf16*)both, D);
+  else
+    return YALM_ERR_DTYPE;
   return launch_status();
 }

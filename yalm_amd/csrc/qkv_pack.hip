@@ -7,6 +7,10 @@
 //   q <- q * (1 + coef ln(floor((p + 1) / every) + 1)) * q_scale      (every 0: no factor)
 //   k likewise with w_k (no factor);  v = qkv[Q + K:] + b_v
 //   blend 1: v_first <- v;   blend 2: v <- (1 - lam) v + lam v_first      (lam a number on the device)
+// head_norm: the norms run a head at a time instead (over the head's d elements, w_q and w_k of d elements shared by
+// the heads).  v_from_k: the product has no value part; a head's values are its keys as projected, before their norm
+// (dv = d).  rot_dims > 0: behind the norms, of each query and key head's first rot_dims elements the neighbours (2p,
+// 2p + 1) are turned by the angle of pair p at the token's position (cos_sin [positions][rot_dims / 2]).
 // Heads are written `pad` elements wide (key size d and value size dv may differ; zeros behind): q_out [T, heads,
 // pad], keys into their page and the step's staging tile [row][pad], values transposed [pad][row].
 #include "common.h"
@@ -23,11 +27,13 @@ __global__ __launch_bounds__(PACK_THREADS) void qkv_pack_kernel(
     const int* __restrict__ seq_tile0, T* __restrict__ k_pages, T* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, int ring_pages, const int* __restrict__ tok_seq,
     const int* __restrict__ tok_pos, const int* __restrict__ seq_slot, const int* __restrict__ seq_len, int n_heads,
-    int n_kv_heads, int d, int dv, int pad, int n_pages, int page_layout, T* __restrict__ v_rows) {
-  extern __shared__ float row[];                  // [Q + K + V]
+    int n_kv_heads, int d, int dv, int pad, int n_pages, int page_layout, T* __restrict__ v_rows, int head_norm,
+    int v_from_k, const float2* __restrict__ cos_sin, int rot_dims, int n_positions) {
+  extern __shared__ float row[];                  // [Q + K + V], then a factor for every query and key head
   __shared__ float red[PACK_THREADS / WAVE];
   const int t = blockIdx.x, tid = threadIdx.x;
-  const int Q = n_heads * d, K = n_kv_heads * d, V = n_kv_heads * dv, N = Q + K + V;
+  const int Q = n_heads * d, K = n_kv_heads * d, V = n_kv_heads * dv, N = Q + K + (v_from_k ? 0 : V);
+  float* head_f = row + N;                        // head_norm: 1 / rms of each query head, then of each key head
   const float* src = qkv + (size_t)t * N;
   float sq = 0.f, sk = 0.f;
 #pragma unroll 4
@@ -40,18 +46,37 @@ __global__ __launch_bounds__(PACK_THREADS) void qkv_pack_kernel(
   sq = block_sum<PACK_THREADS / WAVE>(sq, red);
   sk = block_sum<PACK_THREADS / WAVE>(sk, red);
   __syncthreads();
+  if (head_norm) {                                // a wave a head: the sum of its squares
+    for (int hh = tid / WAVE; hh < n_heads + n_kv_heads; hh += PACK_THREADS / WAVE) {
+      float s = 0.f;
+      for (int e = tid % WAVE; e < d; e += WAVE) s = fmaf(row[hh * d + e], row[hh * d + e], s);
+      s = wave_sum(s);
+      if (tid % WAVE == 0) head_f[hh] = 1.0f / sqrtf(s / (float)d + eps);
+    }
+    __syncthreads();
+  }
   const int pos = tok_pos[t];
+  const float2* cs = rot_dims > 0 ? cos_sin + (size_t)min(max(pos, 0), n_positions - 1) * (rot_dims / 2) : nullptr;
   const int b = tok_seq[t];
   const int slot = b >= 0 ? seq_slot[b] : -1;
 
   // the queries
   float fq = q_scale;
-  if (w_q != nullptr) fq *= 1.0f / sqrtf(sq / (float)Q + eps);
+  if (w_q != nullptr && !head_norm) fq *= 1.0f / sqrtf(sq / (float)Q + eps);
   if (temp_every > 0) fq *= 1.0f + temp_coef * logf((float)((pos + 1) / temp_every) + 1.0f);
   for (int i = tid; i < n_heads * pad; i += PACK_THREADS) {
     const int h = i / pad, e = i - h * pad;
     float v = 0.f;
-    if (e < d) v = row[h * d + e] * fq * (w_q != nullptr ? w_q[h * d + e] : 1.0f);
+    if (e < d) {
+      const float f = head_norm && w_q != nullptr ? fq * head_f[h] : fq;
+      auto normed = [&](int el) { return row[h * d + el] * f * (w_q != nullptr ? w_q[head_norm ? el : h * d + el] : 1.0f); };
+      v = normed(e);
+      if (e < rot_dims) {
+        const float2 c = cs[e >> 1];
+        const float other = normed(e ^ 1);
+        v = (e & 1) ? fmaf(v, c.x, other * c.y) : fmaf(v, c.x, -other * c.y);
+      }
+    }
     q_out[(size_t)t * n_heads * pad + i] = from_f32<T>(v);
   }
 
@@ -67,14 +92,23 @@ __global__ __launch_bounds__(PACK_THREADS) void qkv_pack_kernel(
   }
   if (k_stage != nullptr && b >= 0 && pos >= 0) tile = (long)seq_tile0[b] + pos / PAGE;
 
-  const float fk = w_k != nullptr ? 1.0f / sqrtf(sk / (float)K + eps) : 1.0f;
+  const float fk = w_k != nullptr && !head_norm ? 1.0f / sqrtf(sk / (float)K + eps) : 1.0f;
   const float lam = blend == 2 ? lam_p[0] : 0.f;
   for (int i = tid; i < n_kv_heads * pad; i += PACK_THREADS) {
     const int g = i / pad, e = i - g * pad;
     float kv = 0.f, vv = 0.f;
-    if (e < d) kv = row[Q + g * d + e] * fk * (w_k != nullptr ? w_k[g * d + e] : 1.0f);
+    if (e < d) {
+      const float f = head_norm && w_k != nullptr ? head_f[n_heads + g] : fk;
+      auto normed = [&](int el) { return row[Q + g * d + el] * f * (w_k != nullptr ? w_k[head_norm ? el : g * d + el] : 1.0f); };
+      kv = normed(e);
+      if (e < rot_dims) {
+        const float2 c = cs[e >> 1];
+        const float other = normed(e ^ 1);
+        kv = (e & 1) ? fmaf(kv, c.x, other * c.y) : fmaf(kv, c.x, -other * c.y);
+      }
+    }
     if (e < dv) {
-      vv = row[Q + K + g * dv + e];
+      vv = v_from_k ? row[Q + g * d + e] : row[Q + K + g * dv + e];
       float* first = v_first != nullptr ? v_first + (size_t)t * V + g * dv + e : nullptr;
       if (blend == 1) *first = vv;
       else if (blend == 2) vv = (1.0f - lam) * vv + lam * *first;
@@ -323,20 +357,24 @@ extern "C" int yalm_qkv_pack(const float* qkv, const float* bias, const float* w
                              void* k_pages, void* v_pages, const int* block_table, int table_stride, int ring_pages,
                              const int* tok_seq, const int* tok_pos, const int* seq_slot, const int* seq_len, int T,
                              int n_heads, int n_kv_heads, int d, int dv, int pad, int n_pages, int page_layout,
-                             int dtype, void* v_rows, hipStream_t stream) {
+                             int dtype, void* v_rows, int head_norm, int v_from_k, const float* cos_sin, int rot_dims,
+                             int n_positions, hipStream_t stream) {
   if (T <= 0) return YALM_OK;
+  if ((v_from_k && (d != dv || blend != 0)) || rot_dims < 0 || rot_dims % 2 || rot_dims > d ||
+      (rot_dims > 0 && (cos_sin == nullptr || n_positions <= 0)))
+    return YALM_ERR_ARG;
   if (n_heads <= 0 || n_kv_heads <= 0 || d <= 0 || dv <= 0 || pad < d || pad < dv || temp_every < 0 || blend < 0 ||
       blend > 2 || (blend != 0 && v_first == nullptr) || (blend == 2 && lam == nullptr) ||
       (k_stage != nullptr && (v_stage == nullptr || seq_tile0 == nullptr)) ||
       (k_pages != nullptr && (v_pages == nullptr || block_table == nullptr || ring_pages <= 0 || seq_len == nullptr)) ||
       !page_layout_ok(page_layout, pad))
     return YALM_ERR_ARG;
-  const size_t lds = (size_t)(n_heads * d + n_kv_heads * (d + dv)) * sizeof(float);
+  const int n_row = n_heads * d + n_kv_heads * (d + (v_from_k ? 0 : dv));
+  const size_t lds = (size_t)(n_row + n_heads + n_kv_heads) * sizeof(float);
   if (lds > 64 * 1024) return YALM_ERR_ARG;
-  const int n_row = n_heads * d + n_kv_heads * (d + dv);
   // a wave a token where a lane can take four elements at a time and the row fits its registers, and where the tokens
   // are many: a few tokens are done sooner by 1,024 threads each (8 tokens of 6,144 numbers: 12 against 25 us)
-  const bool by_wave = T >= 32 && d % 4 == 0 && dv % 4 == 0 && n_row <= 256 * 32 &&
+  const bool by_wave = !head_norm && !v_from_k && rot_dims == 0 && T >= 32 && d % 4 == 0 && dv % 4 == 0 && n_row <= 256 * 32 &&
                        ((((uintptr_t)qkv) | ((uintptr_t)bias) | ((uintptr_t)w_q) | ((uintptr_t)w_k) | ((uintptr_t)v_first) |
                          ((uintptr_t)q_out) | ((uintptr_t)k_stage) | ((uintptr_t)k_pages) | ((uintptr_t)v_rows)) & 15) == 0;
   if (by_wave) {
@@ -370,7 +408,8 @@ extern "C" int yalm_qkv_pack(const float* qkv, const float* bias, const float* w
   qkv_pack_kernel<TYPE, NT><<<T, NT, lds, stream>>>(                                                                 \
       qkv, bias, w_q, w_k, eps, temp_coef, temp_every, q_scale, v_first, blend, lam, (TYPE*)q_out, (TYPE*)k_stage,    \
       (TYPE*)v_stage, seq_tile0, (TYPE*)k_pages, (TYPE*)v_pages, block_table, table_stride, ring_pages, tok_seq,     \
-      tok_pos, seq_slot, seq_len, n_heads, n_kv_heads, d, dv, pad, n_pages, page_layout, (TYPE*)v_rows)
+      tok_pos, seq_slot, seq_len, n_heads, n_kv_heads, d, dv, pad, n_pages, page_layout, (TYPE*)v_rows, head_norm,    \
+      v_from_k, (const float2*)cos_sin, rot_dims, n_positions)
   if (dtype == YALM_F32) {
     YALM_PACK(float);
   } else if (dtype == YALM_BF16) {

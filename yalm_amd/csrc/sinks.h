@@ -8,8 +8,9 @@
 
 // What shapes a score between the product q . k / sqrt(head size) and the softmax, beside the mask: a cap
 // (score <- cap tanh(score / cap); 0: none), then a term by the distance of query and key, bias[head][min(distance,
-// n_bias - 1)] (null: none) and/or -slope[head] * distance (null: none), and a logit per head that stands in the
-// softmax's denominator without a key or a value of its own (sink_logit[head], null: none; it enters as it is).
+// n_bias - 1)] (null: none) and/or -slope[head] * distance (null: none) and/or -log_a[head] * ln(1 + log_b[head] *
+// distance) (null: none), and a logit per head that stands in the softmax's denominator without a key or a value of
+// its own (sink_logit[head], null: none; it enters as it is).
 struct ScoreShape {
   const float* bias;
   int n_bias;
@@ -17,8 +18,10 @@ struct ScoreShape {
   const float* sink_logit;
   const float* slope;
   int block;                  // part of the mask: a query sees the keys of its own block of `block` positions only (0: no blocks)
+  const float* log_a;         // [heads], with log_b [heads]: the term that grows with the distance's logarithm
+  const float* log_b;
   __host__ __device__ bool any() const {
-    return bias != nullptr || softcap > 0.f || sink_logit != nullptr || slope != nullptr;
+    return bias != nullptr || softcap > 0.f || sink_logit != nullptr || slope != nullptr || log_a != nullptr;
   }
 };
 // The first position that a query at `pos` sees: not behind a window of `window` keys (0: none) and not before the start
@@ -27,6 +30,11 @@ __host__ __device__ __forceinline__ int first_visible(int pos, int window, int b
   int lo = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
   if (block > 0 && pos / block * block > lo) lo = pos / block * block;
   return lo;
+}
+// -a log2(1 + b distance): the logarithmic term of a score counted in exponents of 2 (-a ln(1 + b distance) in
+// natural units), from the logarithm instruction
+__device__ __forceinline__ float log_distance_term2(float a, float b, int dist) {
+  return -a * __builtin_amdgcn_logf(fmaf(b, (float)max(dist, 0), 1.0f));
 }
 // cap tanh(s / cap) from the exponential instruction (the matrix-core kernels; absolute error about 1e-7 cap)
 __device__ __forceinline__ float soft_cap_fast(float s, float cap) {

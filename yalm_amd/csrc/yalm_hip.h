@@ -176,13 +176,15 @@ int yalm_attn_prefill_lse(const void* q, const void* k_stage, const void* v_stag
                           const int* cu_seqlens, const int* seq_tile0, const int* tok_seq, const int* tok_pos,
                           const int* tile_order, int n_order, int T, int B, int n_tiles, int n_heads, int n_kv_heads,
                           int head_dim, int window, int dtype, int force_simple, const float* score_bias, int n_bias,
-                          float softcap, const float* sink_logit, const float* slopes, int block, hipStream_t stream);
+                          float softcap, const float* sink_logit, const float* slopes, int block, const float* log_a,
+                          const float* log_b, hipStream_t stream);
 int yalm_attn_decode_lse(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
                          int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
                          float* lse, float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
                          int n_splits, int n_pages, int page_layout, int dtype, int force_simple,
                          const int* step_max_len, const int* seq_order, const float* score_bias, int n_bias,
-                         float softcap, const float* sink_logit, const float* slopes, int block, hipStream_t stream);
+                         float softcap, const float* sink_logit, const float* slopes, int block, const float* log_a,
+                          const float* log_b, hipStream_t stream);
 
 // Attention sinks beside a window (src/infer.cpp:305-319, 486-488): the first n_sinks positions of a
 // sequence stay visible when the window has moved past them, and each then counts as lying
@@ -318,13 +320,18 @@ int yalm_embed_sinusoid(const void* table, int table_dtype, const int* tokens, c
 // ln(floor((p + 1) / temp_every) + 1); blend 1 stores the values in v_first (float32 [T, G dv]), blend 2 replaces them
 // by (1 - lam) v + lam v_first (lam: one float32 on the device).  Heads are written `pad` wide with zeros behind
 // (pad >= d, dv): q_out [T, H, pad]; keys and values into the cache pages (page_layout of head size pad) and, with
-// k_stage, into the staging tiles of a step of whole prompts, as yalm_rope_kv_write does.
+// k_stage, into the staging tiles of a step of whole prompts, as yalm_rope_kv_write does.  head_norm != 0: the norms run
+// over each head's d elements instead, with w_q and w_k of d elements shared by the heads.  v_from_k != 0: qkv has no value
+// part, [T, H d + G d], and a head's values are its keys as projected, before their norm (dv = d, no blend).  rot_dims > 0:
+// behind the norms, the neighbours (2p, 2p + 1), p < rot_dims / 2, of every query and key head are turned by the angle
+// cos_sin[position][p] ((cos, sin) float32 [n_positions, rot_dims / 2, 2]).
 int yalm_qkv_pack(const float* qkv, const float* bias, const float* w_q, const float* w_k, float eps, float temp_coef,
                   int temp_every, float q_scale, float* v_first, int blend, const float* lam, void* q_out, void* k_stage,
                   void* v_stage, const int* seq_tile0, void* k_pages, void* v_pages, const int* block_table,
                   int table_stride, int ring_pages, const int* tok_seq, const int* tok_pos, const int* seq_slot,
                   const int* seq_len, int T, int n_heads, int n_kv_heads, int d, int dv, int pad, int n_pages,
-                  int page_layout, int dtype, void* v_rows, hipStream_t stream);
+                  int page_layout, int dtype, void* v_rows, int head_norm, int v_from_k, const float* cos_sin, int rot_dims,
+                  int n_positions, hipStream_t stream);
 // v_rows (`dtype` [T, G, pad]; may be null): yalm_qkv_pack then leaves the values there row by row instead of in their
 // transposed places, and yalm_v_tiles brings them into v_stage [n_tiles, G, pad, 64] and the cache pages (v_pages null:
 // none) a tile of 64 tokens at a time through LDS (pad a multiple of 16; 64 (pad + 8) elements must fit 64 KB).
@@ -378,6 +385,29 @@ int yalm_activate(const float* z, void* out, long n, int kind, int out_dtype, hi
 // x[t, :] (+)= sigmoid(h[t, :] . w) * y[t, :]; h [T, D] and w [D] of `dtype`, x and y float32; accumulate 0: x is written.
 int yalm_gated_add(const float* y, const void* h, const void* w, int dtype, float* x, int T, int D, int accumulate,
                    hipStream_t stream);
+// out[t, c] = (residual ? h[t, c] : 0) + sum_j w[c, j] in(t - (taps - 1) + j, c): a causal convolution over the tokens of
+// each sequence (h, out [T, D] of `dtype`, not the same memory; w float32 [D, taps], the last tap on the token itself).
+// carried, float32 [n_slots, taps - 1, D], holds each sequence's last taps - 1 inputs (the newest last): read for the
+// places in front of the step's first token, then left advanced.  Rows of padding (slot -1) read zeros and keep nothing.
+int yalm_time_conv(const void* h, const float* w, float* carried, void* out, const int* tok_seq, const int* cu_seqlens,
+                   const int* seq_slot, int T, int B, int D, int taps, int residual, int dtype, hipStream_t stream);
+// out[t, i] = act(z[t, i] + bias[i]) * (z[t, F + i] + bias[F + i]), i < F: z float32 [T, 2 F] (gate | up), bias float32
+// [2 F] or null, out of `out_dtype`, kind as yalm_activate; with x_bias (float32 [D]) also x[t, :] += x_bias (x float32 [T, D]).
+int yalm_gated_bias_act(const float* z, const float* bias, void* out, int T, int F, int kind, int out_dtype, float* x,
+                        const float* x_bias, int D, hipStream_t stream);
+// o[t, h, e] *= sigmoid(g[t * g_stride + h * dv + e]), e < dv: o of `dtype` [T, n_heads, pad], g float32.
+int yalm_sigmoid_gate(void* o, const float* g, long g_stride, int T, int n_heads, int dv, int pad, int dtype,
+                      hipStream_t stream);
+// both[t] = [x[t] | x0[t]] (`dtype` [T, 2 D]), then x[t] = start (x, x0 float32 [T, D], start float32 [D]).
+int yalm_loop_pack(float* x, const float* x0, const float* start, void* both, int T, int D, int dtype, hipStream_t stream);
+// The HGRN2 recurrence (hgrn2.hip): proj float32 [T, 2 H d + H dv] = z_q | z_f | v of every token; q = silu(z_q), f =
+// lower + (1 - lower) sigmoid(z_f + f_bias) (f_bias, lower float32 [H d]); per head S <- diag(f) S + (1 - f) v^T, o = S^T q;
+// out (`out_dtype` [T, H dv]) = o over its root mean square a head, times w_norm (float32 [dv]).  state float32 [n_slots, H,
+// dv, d] (a head's S column by column), read and left advanced; raw float32 [T, H dv] scratch; the tokens of sequence b are
+// cu_seqlens[b] .. cu_seqlens[b + 1] - 1, in order; a sequence with slot -1 touches no state and gives zeros.  d <= 256.
+int yalm_hgrn2(const float* proj, const float* f_bias, const float* lower, const float* w_norm, float* state, float* raw,
+               const int* cu_seqlens, const int* seq_slot, void* out, int T, int B, int n_heads, int d, int dv, float eps,
+               int out_dtype, hipStream_t stream);
 
 // Yardsticks for the measurement (probes.hip): a kernel that only reads `bytes` bytes once with `workgroups`
 // workgroups (out: 1,024 words of scratch), and a loop of matrix-core instructions on registers (shape 32:

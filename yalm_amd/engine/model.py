@@ -124,8 +124,12 @@ class Model:
         out = {}
         for e in self.schedule:
             if e.writes_cache:
-                mixer = getattr(self.blocks[e.layer], "mixer", None)     # a block without a mixer keeps nothing
-                out[e.cache] = mixer.cache_request() if mixer is not None else None
+                block = self.blocks[e.layer]
+                if hasattr(block, "cache_request"):                      # the block speaks for all its members
+                    out[e.cache] = block.cache_request()
+                else:
+                    mixer = getattr(block, "mixer", None)                # a block without a mixer keeps nothing
+                    out[e.cache] = mixer.cache_request() if mixer is not None else None
         return out
 
     def prepare(self, n_positions):

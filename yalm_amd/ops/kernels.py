@@ -580,6 +580,16 @@ def _bias(score_bias, n_heads):
     return _need(score_bias, "score_bias", torch.float32, (n_heads, n)), n
 
 
+def _log_distance(log_distance, n_heads):
+    """(address of a, address of b) of a term that grows with the logarithm of the distance: log_distance = (a, b), two
+    float32 [n_heads] on the device, adds -a[head] * ln(1 + b[head] * (query position - key position)) to every score
+    (behind the cap); None: no such term."""
+    if log_distance is None:
+        return None, None
+    a, b = log_distance
+    return _need(a, "log_distance a", torch.float32, (n_heads,)), _need(b, "log_distance b", torch.float32, (n_heads,))
+
+
 def _shape(softcap, sink_logit, n_heads, slopes=None):
     """(cap, address of the sink logits, address of the slopes): softcap > 0 replaces every scaled score s by softcap
     tanh(s / softcap) before the score bias; sink_logit, float32 [n_heads] on the device, puts one more term exp(sink_logit[head]) into the
@@ -594,13 +604,13 @@ def _shape(softcap, sink_logit, n_heads, slopes=None):
 
 def attn_prefill(q, k_stage, v_stage, out, cu_seqlens, seq_tile0, tok_seq, tok_pos, n_heads, n_kv_heads, head_dim,
                  window, tile_order=None, lse=None, out_f32=None, score_bias=None, softcap=0.0, sink_logit=None, slopes=None,
-                 block=0):
+                 block=0, log_distance=None):
     """Causal (and windowed) attention of packed sequences that start at position 0, over
     the keys and values that rope_kv_write staged for this step.  tile_order (device int32,
     from prefill_tile_order) only changes the order of the work.  lse (float32 [T, n_heads], optional)
     receives the logarithm of every query's sum of exp(score), for attn_sink_mix; out_f32 (float32 [T, n_heads *
     head_dim], optional) the result before it is rounded to out's dtype, for the same.  score_bias: see _bias;
-    softcap, sink_logit: see _shape.  block > 0: a query sees only the keys of its own block of `block` positions
+    softcap, sink_logit: see _shape; log_distance: see _log_distance.  block > 0: a query sees only the keys of its own block of `block` positions
     (blocks counted from position 0 of its sequence), beside what the window says."""
     if block < 0:
         raise ValueError("a block of positions has a positive size (0: none)")
@@ -627,7 +637,7 @@ def attn_prefill(q, k_stage, v_stage, out, cu_seqlens, seq_tile0, tok_seq, tok_p
                                                       T, B, n_tiles, n_heads, n_kv_heads, head_dim, int(window),
                                                       dtype_code(dt), 1 if FORCE_SIMPLE else 0,
                                                       *_bias(score_bias, n_heads), *_shape(softcap, sink_logit, n_heads, slopes),
-                                                      int(block), _stream()),
+                                                      int(block), *_log_distance(log_distance, n_heads), _stream()),
                   "attn_prefill")
     return out
 
@@ -638,7 +648,7 @@ def attn_decode_workspace_floats(B, n_heads, head_dim, n_splits):
 
 def attn_decode(q, k_pages, v_pages, block_table, ring_pages, seq_slot, seq_len, out, partial, n_heads, n_kv_heads,
                 head_dim, window, n_splits, lse=None, sinks=None, layout=None, step_max_len=None, seq_order=None,
-                score_bias=None, softcap=0.0, sink_logit=None, slopes=None, block=0):
+                score_bias=None, softcap=0.0, sink_logit=None, slopes=None, block=0, log_distance=None):
     """One query per sequence over the cache pages (laid out as `layout` says, default page_layout(head_dim));
     seq_len counts the new key.  lse as in attn_prefill.  step_max_len (int32 [1] on the device, optional): the
     length of the step's longest sequence, with which sequences of unequal lengths are cut into splits of equal
@@ -675,11 +685,12 @@ def attn_decode(q, k_pages, v_pages, block_table, ring_pages, seq_slot, seq_len,
         library.check(library.lib().yalm_attn_decode_lse(
             p_q, p_kp, p_vp, p_bt, stride, ring_pages, p_ss, p_sl, p_o, p_lse, p_w, B, n_heads, n_kv_heads, head_dim,
             int(window), int(n_splits), n_pages, _layout(layout, head_dim), dtype_code(dt), force, p_max, p_ord,
-            *_bias(score_bias, n_heads), *_shape(softcap, sink_logit, n_heads, slopes), int(block), _stream()), "attn_decode")
+            *_bias(score_bias, n_heads), *_shape(softcap, sink_logit, n_heads, slopes), int(block),
+            *_log_distance(log_distance, n_heads), _stream()), "attn_decode")
         return out
     if lse is not None:
         raise ValueError("attn_decode leaves no lse when it takes the sinks in itself")
-    if score_bias is not None or softcap or sink_logit is not None or slopes is not None or block:
+    if score_bias is not None or softcap or sink_logit is not None or slopes is not None or block or log_distance is not None:
         raise ValueError("attention sinks are scored without a score bias, a cap or a sink logit: they do not go together")
     sink_k, sink_v, cos_sin, rotary_dim, store = sinks
     n_slots, _, n_sinks, _ = sink_k.shape
@@ -882,17 +893,29 @@ def v_tiles(v_rows, v_stage, v_pages, cu_seqlens, seq_tile0, block_table, ring_p
 
 def qkv_pack(qkv, bias, w_q, w_k, eps, q_temp, q_scale, v_first, blend, lam, q_out, k_stage, v_stage, seq_tile0, k_pages,
              v_pages, block_table, ring_pages, tok_seq, tok_pos, seq_slot, seq_len, n_heads, n_kv_heads, d, dv, pad,
-             v_rows=None):
+             v_rows=None, head_norm=False, v_from_k=False, cos_sin=None, rot_dims=0):
     """From a q/k/v product to an attention without rotation.  qkv float32 [T, H d + G d + G dv] (+ bias, float32 of
     that width or None); RMS norms over the WHOLE query and key projections with the weights w_q [H d], w_k [G d]
     (float32; None: no norm); the queries times q_scale and, with q_temp = (coef, every), times 1 + coef ln(floor((p + 1)
     / every) + 1) at position p; blend 1 stores the values in v_first (float32 [T, G dv]), blend 2 replaces them by
     (1 - lam) v + lam v_first (lam: one float32 on the device).  Heads are written `pad` wide, zeros behind: q_out [T,
     H pad]; keys and values into the cache pages (None: nowhere) and, with k_stage, into the staging tiles of a step of
-    whole prompts.  v_rows ([T, G pad], optional): the values go there row by row instead (v_tiles then transposes them)."""
+    whole prompts.  v_rows ([T, G pad], optional): the values go there row by row instead (v_tiles then transposes them).
+    head_norm: the norms run over each head's d elements instead, w_q and w_k being [d] and shared by the heads.
+    v_from_k: qkv is [T, H d + G d] only and a head's values are its keys as projected, before their norm (dv = d).
+    rot_dims > 0 with cos_sin (float32 [positions, rot_dims / 2, 2]): behind the norms the neighbours (2p, 2p + 1) of
+    every query and key head's first rot_dims elements are turned by the angle of pair p at the token's position."""
     T = qkv.shape[0]
     Q, K, V = n_heads * d, n_kv_heads * d, n_kv_heads * dv
-    N = Q + K + V
+    N = Q + K + (0 if v_from_k else V)
+    if v_from_k and (d != dv or blend):
+        raise ValueError("qkv_pack: values taken from the keys are as wide as the keys, and are not blended")
+    rot_dims = int(rot_dims or 0)
+    n_pos = 0
+    if rot_dims:
+        if rot_dims % 2 or rot_dims > d or cos_sin is None:
+            raise ValueError("qkv_pack: %d turned elements do not fit heads of %d, or the table of angles is missing" % (rot_dims, d))
+        n_pos = cos_sin.shape[0]
     dt = q_out.dtype
     if pad < max(d, dv) or N * 4 > 64 * 1024:
         raise ValueError("qkv_pack: heads of %d and %d do not fit %d, or a row of %d values is too wide" % (d, dv, pad, N))
@@ -908,7 +931,8 @@ def qkv_pack(qkv, bias, w_q, w_k, eps, q_temp, q_scale, v_first, blend, lam, q_o
             raise ValueError("ring_pages %d does not fit the block table (%d columns)" % (ring_pages, stride))
     library.check(library.lib().yalm_qkv_pack(
         _need(qkv, "qkv", torch.float32, (T, N)), _opt(bias, "bias", torch.float32, (N,)),
-        _opt(w_q, "w_q", torch.float32, (Q,)), _opt(w_k, "w_k", torch.float32, (K,)), float(eps), float(coef), int(every),
+        _opt(w_q, "w_q", torch.float32, (d if head_norm else Q,)), _opt(w_k, "w_k", torch.float32, (d if head_norm else K,)),
+        float(eps), float(coef), int(every),
         float(q_scale), _opt(v_first, "v_first", torch.float32, (T, V)), int(blend), _opt(lam, "lam", torch.float32),
         _need(q_out, "q_out", dt, (T, n_heads * pad)),
         _opt(k_stage, "k_stage", dt, (n_tiles, n_kv_heads, PAGE, pad)),
@@ -917,7 +941,10 @@ def qkv_pack(qkv, bias, w_q, w_k, eps, q_temp, q_scale, v_first, blend, lam, q_o
         _opt(v_pages, "v_pages", dt, (n_pages, n_kv_heads, pad, PAGE)), _opt(block_table, "block_table", torch.int32, (None, None)),
         stride, int(ring_pages), _need(tok_seq, "tok_seq", torch.int32, (T,)), _need(tok_pos, "tok_pos", torch.int32, (T,)),
         _need(seq_slot, "seq_slot", torch.int32), _opt(seq_len, "seq_len", torch.int32), T, n_heads, n_kv_heads, d, dv, pad,
-        n_pages, page_layout(pad), dtype_code(dt), _opt(v_rows, "v_rows", dt, (T, n_kv_heads * pad)), _stream()), "qkv_pack")
+        n_pages, page_layout(pad), dtype_code(dt), _opt(v_rows, "v_rows", dt, (T, n_kv_heads * pad)),
+        1 if head_norm else 0, 1 if v_from_k else 0,
+        _need(cos_sin, "cos_sin", torch.float32, (n_pos, rot_dims // 2, 2)) if rot_dims else None, rot_dims, n_pos,
+        _stream()), "qkv_pack")
     return q_out
 
 
@@ -1057,6 +1084,98 @@ def gated_add(y, h, w, x, accumulate=True):
         _need(y, "y", torch.float32, (T, D)), _need(h, "h", None, (T, D)), _need(w, "w", h.dtype, (D,)), dtype_code(h.dtype),
         _need(x, "x", torch.float32, (T, D)), T, D, 1 if accumulate else 0, _stream()), "gated_add")
     return x
+
+
+TIME_CONV_MAX_TAPS = 16
+
+
+def time_conv(h, w, carried, out, tok_seq, cu_seqlens, seq_slot, residual=True):
+    """out[t, c] = (h[t, c] if residual) + sum_j w[c, j] in(t - (taps - 1) + j, c): a causal convolution over the tokens
+    of each sequence of the step, the last tap on the token itself (h, out [T, D] of one dtype and not the same
+    memory; w float32 [D, taps]).  carried (float32 [slots, taps - 1, D]; None with one tap) holds each sequence's last
+    taps - 1 inputs, read for the places in front of the step's first token and left advanced."""
+    T, D = h.shape
+    taps = w.shape[1]
+    B = seq_slot.shape[0]
+    if not 0 < taps <= TIME_CONV_MAX_TAPS:
+        raise ValueError("time_conv: %d taps (at most %d)" % (taps, TIME_CONV_MAX_TAPS))
+    if h.data_ptr() == out.data_ptr():
+        raise ValueError("time_conv: the result needs memory of its own")
+    p_c = None
+    if taps > 1:
+        p_c = _need(carried, "carried", torch.float32, (None, taps - 1, D))
+    library.check(library.lib().yalm_time_conv(
+        _need(h, "h", None, (T, D)), _need(w, "w", torch.float32, (D, taps)), p_c, _need(out, "out", h.dtype, (T, D)),
+        _need(tok_seq, "tok_seq", torch.int32, (T,)), _need(cu_seqlens, "cu_seqlens", torch.int32, (B + 1,)),
+        _need(seq_slot, "seq_slot", torch.int32, (B,)), T, B, D, taps, 1 if residual else 0, dtype_code(h.dtype), _stream()),
+        "time_conv")
+    return out
+
+
+def gated_bias_act(z, bias, out, kind, x=None, x_bias=None):
+    """out[t, i] = act(z[t, i] + bias[i]) * (z[t, F + i] + bias[F + i]): z float32 [T, 2 F] (gate | up), bias float32
+    [2 F] or None, out [T, F] of its own dtype; kind as in activate.  With x (float32 [T, D]) and x_bias (float32 [D])
+    also x[t] += x_bias."""
+    if kind not in ACTIVATIONS:
+        raise ValueError("activation %r is not offered (%s)" % (kind, ", ".join(ACTIVATIONS)))
+    T, F2 = z.shape
+    F = F2 // 2
+    D = 0
+    p_x = p_xb = None
+    if x_bias is not None:
+        D = x.shape[1]
+        p_x, p_xb = _need(x, "x", torch.float32, (T, D)), _need(x_bias, "x_bias", torch.float32, (D,))
+    library.check(library.lib().yalm_gated_bias_act(
+        _need(z, "z", torch.float32, (T, 2 * F)), _opt(bias, "bias", torch.float32, (2 * F,)), _need(out, "out", None, (T, F)),
+        T, F, ACTIVATIONS[kind], dtype_code(out.dtype), p_x, p_xb, D, _stream()), "gated_bias_act")
+    return out
+
+
+def sigmoid_gate(o, g, n_heads, dv, pad):
+    """o[t, h, e] *= sigmoid(g[t, h dv + e]) for e < dv: o [T, n_heads pad] in its own dtype, g float32 rows of a wider
+    float32 matrix (a view whose rows are g.stride(0) apart)."""
+    T = o.shape[0]
+    if g.dtype != torch.float32 or g.dim() != 2 or g.shape != (T, n_heads * dv) or g.stride(1) != 1 or not g.is_cuda:
+        raise ValueError("sigmoid_gate: the gates are float32 [%d, %d] on the device, rows contiguous" % (T, n_heads * dv))
+    library.check(library.lib().yalm_sigmoid_gate(
+        _need(o, "o", None, (T, n_heads * pad)), g.data_ptr(), int(g.stride(0)), T, n_heads, dv, pad, dtype_code(o.dtype),
+        _stream()), "sigmoid_gate")
+    return o
+
+
+def loop_pack(x, x0, start, both):
+    """both[t] = [x[t] | x0[t]] in both's dtype, then x[t] = start (x, x0 float32 [T, D]; start float32 [D])."""
+    T, D = x.shape
+    library.check(library.lib().yalm_loop_pack(
+        _need(x, "x", torch.float32, (T, D)), _need(x0, "x0", torch.float32, (T, D)), _need(start, "start", torch.float32, (D,)),
+        _need(both, "both", None, (T, 2 * D)), T, D, dtype_code(both.dtype), _stream()), "loop_pack")
+    return both
+
+
+HGRN2_MAX_KEY_DIM = 256           # a lane of the recurrence holds 32 rows of a state column at most
+
+
+def hgrn2_state_elements(n_heads, d, dv):
+    return n_heads * d * dv
+
+
+def hgrn2(proj, f_bias, lower, w_norm, state, raw, cu_seqlens, seq_slot, out, n_heads, d, dv, eps):
+    """The HGRN2 recurrence over a step's tokens.  proj float32 [T, 2 H d + H dv] = z_q | z_f | v; q = silu(z_q), f = lower
+    + (1 - lower) sigmoid(z_f + f_bias); per head S <- diag(f) S + (1 - f) v^T, o = S^T q; out [T, H dv] = o over its root
+    mean square a head, times w_norm [dv].  state float32 [slots, H dv d] (a head's S column by column) is read and left
+    advanced; raw float32 [T, H dv] is scratch.  Sequence b's tokens are cu_seqlens[b] .. cu_seqlens[b + 1] - 1."""
+    T = proj.shape[0]
+    B = seq_slot.shape[0]
+    N = 2 * n_heads * d + n_heads * dv
+    if not 0 < d <= HGRN2_MAX_KEY_DIM:
+        raise ValueError("hgrn2: key heads of %d (at most %d)" % (d, HGRN2_MAX_KEY_DIM))
+    library.check(library.lib().yalm_hgrn2(
+        _need(proj, "proj", torch.float32, (T, N)), _need(f_bias, "f_bias", torch.float32, (n_heads * d,)),
+        _need(lower, "lower", torch.float32, (n_heads * d,)), _need(w_norm, "w_norm", torch.float32, (dv,)),
+        _need(state, "state", torch.float32, (None, n_heads * d * dv)), _need(raw, "raw", torch.float32, (T, n_heads * dv)),
+        _need(cu_seqlens, "cu_seqlens", torch.int32, (B + 1,)), _need(seq_slot, "seq_slot", torch.int32, (B,)),
+        _need(out, "out", None, (T, n_heads * dv)), T, B, n_heads, d, dv, float(eps), dtype_code(out.dtype), _stream()), "hgrn2")
+    return out
 
 
 # ---------------------------------------------------------------------------------------------------------------

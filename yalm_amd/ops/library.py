@@ -34,9 +34,9 @@ _SIGNATURES = {
     "yalm_attn_decode": (_I, [_P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_attn_decode_workspace": (ctypes.c_long, [_I, _I, _I, _I]),
     "yalm_attn_prefill_lse": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I,
-                                   _P, _I, _F, _P, _P, _I, _P]),
+                                   _P, _I, _F, _P, _P, _I, _P, _P, _P]),
     "yalm_attn_decode_lse": (_I, [_P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P,
-                                  _P, _I, _F, _P, _P, _I, _P]),
+                                  _P, _I, _F, _P, _P, _I, _P, _P, _P]),
     "yalm_sink_store": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_attn_sink_mix": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_attn_decode_sinks": (_I, [_P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P]),
@@ -64,7 +64,7 @@ _SIGNATURES = {
     "yalm_moe_grouped": (_I, [_P, _P, _P, _P, _P, _P, _F, _F, _F, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_embed_sinusoid": (_I, [_P, _I, _P, _P, _P, _F, _P, _I, _I, _I, _P]),
     "yalm_qkv_pack": (_I, [_P, _P, _P, _P, _F, _F, _I, _F, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P,
-                           _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P]),
+                           _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _I, _I, _P, _I, _I, _P]),
     "yalm_v_tiles": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_mlstm_chunks": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _F, _F, _F, _I, _I, _I, _P]),
     "yalm_mlstm_chunks_lds": (ctypes.c_long, [_I, _I]),
@@ -73,11 +73,16 @@ _SIGNATURES = {
     "yalm_embed_learned": (_I, [_P, _P, _I, _P, _P, _F, _P, _I, _I, _I, _I, _P]),
     "yalm_activate": (_I, [_P, _P, ctypes.c_long, _I, _I, _P]),
     "yalm_gated_add": (_I, [_P, _P, _P, _I, _P, _I, _I, _I, _P]),
+    "yalm_time_conv": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]),
+    "yalm_gated_bias_act": (_I, [_P, _P, _P, _I, _I, _I, _I, _P, _P, _I, _P]),
+    "yalm_sigmoid_gate": (_I, [_P, _P, ctypes.c_long, _I, _I, _I, _I, _I, _P]),
+    "yalm_loop_pack": (_I, [_P, _P, _P, _P, _I, _I, _I, _P]),
+    "yalm_hgrn2": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P]),
     "yalm_probe_read": (_I, [_P, ctypes.c_long, _P, _I, _P]),
     "yalm_probe_mfma": (_I, [_I, _I, _I, _P, _P, _P]),
 }
 
-ABI_VERSION = 33
+ABI_VERSION = 34
 
 
 class KernelError(RuntimeError):

@@ -8,7 +8,9 @@ it is in.  Kinds of parts and the methods each must have:
   position       prepare(n_positions, device); used by the mixers that name it (one instance per distinct
                  PartSpec of a model if the class says `share_by_spec = True`: it then has no tensors
                  of its own and its prefix means nothing)
-  mixer          cache_request() -> KVRequest | StateRequest | None
+  mixer          cache_request() -> KVRequest | StateRequest | None, or {name: request}: a mixer made of several gets
+                 the cache line (line, name) for each of them
+  input_filter   cache_request() as a mixer's; forward(h[T, dim], out[T, dim], ctx, line): what a sublayer reads in h's place
                  forward(h[T, dim], x_f32[T, dim], ctx, line, writes_cache): adds its output to x
   feed_forward   forward(h[T, dim], x_f32[T, dim], ctx): adds its output to x
   block          forward(x_f32[T, dim], ctx, line, writes_cache): one layer on the residual stream;
@@ -41,7 +43,7 @@ from typing import Callable, Dict, List
 from ..config.spec import PartSpec
 from ..weights.loader import ParamSpec
 
-ROLES = ("norm", "position", "mixer", "feed_forward", "block", "embedding", "head")
+ROLES = ("norm", "position", "mixer", "feed_forward", "block", "embedding", "head", "input_filter")
 _REGISTRY: Dict[str, Dict[str, type]] = {r: {} for r in ROLES}
 
 

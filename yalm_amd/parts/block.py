@@ -17,9 +17,20 @@ class PreNormResidualBlock(Part):
         if layer_spec.part("feed_forward") is not None:
             self.feed_forward_norm = build_part("norm", layer_spec.feed_forward_norm, dim, p)
             self.feed_forward = build_part("feed_forward", layer_spec.feed_forward, dim, p)
+        # optional member mixer_input: a filter between the first norm and the mixer (a short convolution over time)
+        self.mixer_input = None
+        if layer_spec.part("mixer_input") is not None:
+            self.mixer_input = build_part("input_filter", layer_spec.mixer_input, dim, p)
 
     def children(self):
-        return [c for c in (self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward) if c is not None]
+        return [c for c in (self.mixer_norm, self.mixer_input, self.mixer, self.feed_forward_norm, self.feed_forward)
+                if c is not None]
+
+    def cache_request(self):
+        """What the layer keeps for a sequence: the mixer's, and beside it what the filter in front of the mixer keeps."""
+        if self.mixer_input is None:
+            return self.mixer.cache_request()
+        return {"mixer": self.mixer.cache_request(), "input": self.mixer_input.cache_request()}
 
     def first_norm(self):
         """The norm that reads the residual stream first when this layer runs (the layer before
@@ -28,7 +39,18 @@ class PreNormResidualBlock(Part):
 
     def forward(self, x, ctx, line, writes_cache=True, next_norm=None):
         plain_end = False                 # whether the layer's last sublayer ran behind a norm kernel of its own
-        if self.mixer.fuses_norm(self.mixer_norm, x, ctx):
+        if self.mixer_input is not None:
+            left = ctx.normed.pop(id(self.mixer_norm), None)
+            if left is not None and left[1] is None:      # the layer before has left this norm's output
+                h = left[0]
+            else:
+                h = ctx.ws.get("block.h", (x.shape[0], self.dim), ctx.act_dtype)
+                self.mixer_norm.forward(x, h, ctx)
+            filtered = ctx.ws.get("block.filtered", (x.shape[0], self.dim), ctx.act_dtype)
+            self.mixer_input.forward(h, filtered, ctx, (line, "input"))
+            self.mixer.forward(filtered, x, ctx, (line, "mixer"), writes_cache)
+            plain_end = self.feed_forward is None
+        elif self.mixer.fuses_norm(self.mixer_norm, x, ctx):
             self.mixer.forward_prenorm(x, self.mixer_norm, ctx, line, writes_cache,
                                        emit_for=self.feed_forward_norm if self.feed_forward is not None else next_norm)
         else:
@@ -157,3 +179,47 @@ class PostNormResidualBlock(Part):
             self.feed_forward_norm.add_normed(y, x, ctx, h_out=hand_on, next_norm=final)
         if hand_on is not None:
             ctx.normed[id(next_norm)] = (hand_on, None, None)
+
+
+@part("block", "loop_entry")
+class LoopEntryBlock(Part):
+    """The way into a walk of looped layers: x <- W [x; x0] + start, x0 being what the embedding left (it keeps a copy
+    when its `keep_output` is set) and `start` row `walk` of a table [walks, dim].  No mixer and no cache line; the
+    product reads both streams rounded to the compute dtype and adds to the float32 stream, which the packing kernel
+    has set to `start`.  Parameters: `walk`, `walks`, `matrix` and `starts` (tensor names)."""
+
+    def __init__(self, layer_spec, dim, prefix=""):
+        super().__init__(None, dim, layer_spec.prefix)
+        p = layer_spec.entry.params
+        self.walk, self.walks = int(p["walk"]), int(p["walks"])
+        if not 0 <= self.walk < self.walks:
+            raise ValueError("walk %d of %d" % (self.walk, self.walks))
+        self.matrix = self.prefix + str(p.get("matrix", "in"))
+        self.starts = self.prefix + str(p.get("starts", "step"))
+        self.w = self.start = None
+
+    def param_specs(self):
+        from ..weights.loader import ParamSpec
+        return [ParamSpec(self.matrix, (self.dim, 2 * self.dim), fan_in=2 * self.dim),
+                ParamSpec(self.starts, (self.walks, self.dim), init="bias")]
+
+    def load(self, get, compute_dtype, device):
+        import torch
+        from ..weights.loader import place
+        self.w = place(get(self.matrix), compute_dtype, device)
+        self.start = get(self.starts).to(torch.float32)[self.walk].to(device).contiguous()
+
+    def weight_bytes(self):
+        return self.w.numel() * self.w.element_size()
+
+    def first_norm(self):
+        return None
+
+    def forward(self, x, ctx, line, writes_cache=True, next_norm=None):
+        import torch
+        from ..ops import kernels
+        T = x.shape[0]
+        x0 = ctx.ws.get("embed.kept", (T, self.dim), torch.float32)
+        both = ctx.ws.get("loop.both", (T, 2 * self.dim), ctx.act_dtype)
+        kernels.loop_pack(x, x0, self.start, both)
+        self._gemm(ctx, both, self.w, x, kernels.EPI_ADD_F32)

@@ -2,7 +2,7 @@
 when tied (src/model.cpp:389-398); one copy on the device either way."""
 from ..ops import kernels
 from ..weights.loader import ParamSpec, place
-from .base import Part, part
+from .base import Part, build_part, part
 
 
 @part("embedding", "token_embedding")
@@ -10,7 +10,9 @@ class TokenEmbedding(Part):
     """x[t] = float(table[token[t]]) (src/infer.cpp:454-475), times `scale` (default 1), plus, with `sinusoid_base` b,
     a position vector whose entry 2i is sin(p b^(-2i / width)) and whose entry 2i + 1 is the cosine of the same angle
     (the frequencies are made in float64 and the angle is exact at every position), or, with `position_tensor` (a
-    tensor's name) and `n_positions`, plus the row of that learned table [n_positions, width] at the token's position."""
+    tensor's name) and `n_positions`, plus the row of that learned table [n_positions, width] at the token's position.
+    With `norm` (a norm's PartSpec) the result passes that norm at once, in float32; with `keep_output` a copy of what the
+    part leaves stays in the step's buffer "embed.kept" for layers that read it again (the way into looped layers)."""
 
     def __init__(self, spec, dim, prefix):
         super().__init__(spec, dim, prefix)
@@ -25,6 +27,11 @@ class TokenEmbedding(Part):
         self.table = None
         self.freq = None
         self.positions = None
+        self.norm = build_part("norm", spec.params["norm"], dim, prefix) if spec.params.get("norm") else None
+        self.keep_output = bool(spec.params.get("keep_output", False))
+
+    def children(self):
+        return [self.norm] if self.norm is not None else []
 
     def param_specs(self):
         out = [ParamSpec(self.tensor, (self.vocab_size, self.dim), init="embedding")]
@@ -46,6 +53,21 @@ class TokenEmbedding(Part):
         return (2 if self.positions is not None else 1) * self.dim * self.table.element_size()     # one row per token
 
     def forward(self, tokens, x, ctx):
+        import torch
+        kept = ctx.ws.get("embed.kept", tuple(x.shape), torch.float32) if self.keep_output else None
+        if self.norm is None:
+            self._rows(tokens, x, ctx)
+            if kept is not None:
+                self._rows(tokens, kept, ctx)
+            return x
+        raw = ctx.ws.get("embed.raw", tuple(x.shape), torch.float32)
+        self._rows(tokens, raw, ctx)
+        self.norm.forward(raw, x, ctx)
+        if kept is not None:
+            self.norm.forward(raw, kept, ctx)
+        return x
+
+    def _rows(self, tokens, x, ctx):
         if self.positions is not None:
             if ctx.max_position >= self.n_positions:
                 raise ValueError("position %d is beyond the %d rows of the position table" % (ctx.max_position, self.n_positions))
