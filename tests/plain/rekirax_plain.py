@@ -129,20 +129,39 @@ def remember(memory, k, v):
     return keys, values
 
 
-def window_attention(h, positions, mixer, w, prefix, eps, memory):
-    """The mixer 'attention': keys double as values (as projected, before their norm); norms a head; capped scores
-    less r1 ln(1 + r2 distance); a sliding window."""
+def window_projections(h, mixer, w, prefix, eps):
+    """(q [T, H, d] and k [T, G, d], each head normed with a weight of d elements that the heads share; the keys as
+    projected [T, G, d], which are the values)."""
     H, G, d = int(mixer["heads"]), int(mixer["kv_heads"]), int(mixer["dim"])
     T = h.shape[0]
     q = (h @ W(w, prefix + "q").T).reshape(T, H, d)
     k_raw = (h @ W(w, prefix + "k").T).reshape(T, G, d)
-    q = rms_div(q, eps) * W(w, prefix + "q.norm")
-    k = rms_div(k_raw, eps) * W(w, prefix + "k.norm")
+    return rms_div(q, eps) * W(w, prefix + "q.norm"), rms_div(k_raw, eps) * W(w, prefix + "k.norm"), k_raw
+
+
+def chunk_projections(h, positions, mixer, w, prefix, eps):
+    """(q [T, H, d], k [T, G, d], v [T, G, dv]): norms over the whole query and key projections, then the rotation."""
+    H, G, d, dv = int(mixer["heads"]), int(mixer["kv_heads"]), int(mixer["dim"]), int(mixer["vdim"])
+    T = h.shape[0]
+    q = rms_div(h @ W(w, prefix + "q").T, eps) * W(w, prefix + "q.norm")
+    k = rms_div(h @ W(w, prefix + "k").T, eps) * W(w, prefix + "k.norm")
+    v = (h @ W(w, prefix + "v").T).reshape(T, G, dv)
+    rot = mixer.get("rot") or {}
+    dims, base = int(rot.get("dims", 0) or 0), float(rot.get("base", 10000.0))
+    return rotate_half(q.reshape(T, H, d), positions, dims, base), rotate_half(k.reshape(T, G, d), positions, dims, base), v
+
+
+def window_attention(h, positions, mixer, w, prefix, eps, memory):
+    """The mixer 'attention': keys double as values (as projected, before their norm); norms a head; capped scores
+    less r1 ln(1 + r2 distance); a sliding window."""
+    H, d = int(mixer["heads"]), int(mixer["dim"])
+    T = h.shape[0]
+    q, k, k_raw = window_projections(h, mixer, w, prefix, eps)
     keys, values = remember(memory, k, k_raw)
     assert keys.shape[0] == positions[-1] + 1
     cap = float(mixer.get("softcap") or 0.0)
     r1, r2 = W(w, prefix + "r1"), W(w, prefix + "r2")
-    size = int(mixer["mask"]["size"])
+    size = int(mixer["mask"]["size"]) if mixer.get("mask") else 1 << 60
 
     def shape_score(s, hd, dist):
         if cap:
@@ -156,18 +175,12 @@ def window_attention(h, positions, mixer, w, prefix, eps, memory):
 def chunk_attention(h, positions, mixer, w, prefix, eps, memory):
     """The left half of the mixer 'parallel': norms over the whole projections, then rotation of the heads' first
     elements; chunks of positions; the heads times sigmoid(W_g h) before the output projection."""
-    H, G, d, dv = int(mixer["heads"]), int(mixer["kv_heads"]), int(mixer["dim"]), int(mixer["vdim"])
+    H, dv = int(mixer["heads"]), int(mixer["vdim"])
     T = h.shape[0]
-    q = rms_div(h @ W(w, prefix + "q").T, eps) * W(w, prefix + "q.norm")
-    k = rms_div(h @ W(w, prefix + "k").T, eps) * W(w, prefix + "k.norm")
-    v = (h @ W(w, prefix + "v").T).reshape(T, G, dv)
-    rot = mixer.get("rot") or {}
-    dims, base = int(rot.get("dims", 0) or 0), float(rot.get("base", 10000.0))
-    q = rotate_half(q.reshape(T, H, d), positions, dims, base)
-    k = rotate_half(k.reshape(T, G, d), positions, dims, base)
+    q, k, v = chunk_projections(h, positions, mixer, w, prefix, eps)
     keys, values = remember(memory, k, v)
     assert keys.shape[0] == positions[-1] + 1
-    size = int(mixer["mask"]["size"])
+    size = int(mixer["mask"]["size"]) if mixer.get("mask") else 1 << 60
     o = softmax_over_visible(q, keys, values, positions, float(mixer["scale"]), lambda i, j: sees_chunk(i, j, size))
     gate = torch.sigmoid(h @ W(w, prefix + "g").T)
     return (o.reshape(T, H * dv) * gate) @ W(w, prefix + "o").T
@@ -190,7 +203,9 @@ def hgrn2_recurrence(q, f, v, S):
     return o, S
 
 
-def hgrn2(h, mixer, w, prefix, eps, memory):
+def hgrn2(h, mixer, w, prefix, eps, memory, reads_out=None):
+    """reads_out, if a list, receives [T]: the smallest root mean square among the heads' results before their norm,
+    which divides by it (a head that reads next to nothing from its state is normed up from rounding's leavings)."""
     H, d, dv = int(mixer["heads"]), int(mixer["dim"]), int(mixer["vdim"])
     T = h.shape[0]
     q = silu(h @ W(w, prefix + "q").T).reshape(T, H, d)
@@ -200,14 +215,16 @@ def hgrn2(h, mixer, w, prefix, eps, memory):
     if S is None:
         S = torch.zeros((H, d, dv), dtype=F64)
     o, memory["S"] = hgrn2_recurrence(q, f, v, S)
+    if reads_out is not None:
+        reads_out.append(torch.sqrt((o * o).mean(dim=-1)).min(dim=-1).values)
     o = rms_div(o, eps) * W(w, prefix + "norm")
     return o.reshape(T, H * dv) @ W(w, prefix + "o").T
 
 
-def parallel_mixer(h, positions, mixer, w, prefix, eps, memory):
+def parallel_mixer(h, positions, mixer, w, prefix, eps, memory, reads_out=None):
     """Half the sum of the two mixers' results, each normed over the width with a plain weight of its own."""
     left = chunk_attention(h, positions, mixer["left"], w, prefix + "left.", eps, memory.setdefault("left", {}))
-    right = hgrn2(h, mixer["right"], w, prefix + "right.", eps, memory.setdefault("right", {}))
+    right = hgrn2(h, mixer["right"], w, prefix + "right.", eps, memory.setdefault("right", {}), reads_out)
     return 0.5 * (rms_div(left, eps) * W(w, prefix + "left.out") + rms_div(right, eps) * W(w, prefix + "right.out"))
 
 
@@ -219,12 +236,12 @@ def gated_ff(h, w, prefix):
 
 
 # ------------------------------------------------------------------------------------------ the model
-def layer_forward(x, positions, layer, w, p, eps, memory):
+def layer_forward(x, positions, layer, w, p, eps, memory, reads_out=None):
     h = norm_one_plus(x, W(w, p + "norm1"), eps)
     if (p + "canon1") in w:
         h = input_conv(h, W(w, p + "canon1"), memory)
     if layer["type"] == "parallel":
-        y = parallel_mixer(h, positions, layer["mixer"], w, p + "mix.", eps, memory)
+        y = parallel_mixer(h, positions, layer["mixer"], w, p + "mix.", eps, memory, reads_out)
     else:
         y = window_attention(h, positions, layer["mixer"], w, p + "mix.", eps, memory)
     x = x + y
@@ -233,10 +250,11 @@ def layer_forward(x, positions, layer, w, p, eps, memory):
     return x
 
 
-def forward(config, w, tokens, memory=None, start=0, layers_out=None):
+def forward(config, w, tokens, memory=None, start=0, layers_out=None, reads_out=None):
     """Logits [T, vocab] of `tokens` at positions start, start + 1, ... of one sequence; `memory` (a
     dictionary, empty at the sequence's start) carries the layers' keys, values and states from call to
-    call.  layers_out, if a list, receives the residual stream after every run of a layer."""
+    call.  layers_out, if a list, receives the residual stream after every run of a layer; reads_out, if a list,
+    what hgrn2 reports of every run of a recurrent layer."""
     memory = {} if memory is None else memory
     eps = float(config["norm"]["eps"])
     positions = list(range(start, start + len(tokens)))
@@ -246,7 +264,7 @@ def forward(config, w, tokens, memory=None, start=0, layers_out=None):
     for i, t in run_order(len(config["layers"]), loop):
         if loop and i == int(loop["start"]):
             x = loop_entry(x, x0, w, t)
-        x = layer_forward(x, positions, config["layers"][i], w, "l%d." % i, eps, memory.setdefault((i, t), {}))
+        x = layer_forward(x, positions, config["layers"][i], w, "l%d." % i, eps, memory.setdefault((i, t), {}), reads_out)
         if layers_out is not None:
             layers_out.append(x.clone())
     return norm_one_plus(x, W(w, "final.norm"), eps) @ W(w, "embed").T
