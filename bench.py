@@ -8,7 +8,7 @@ shape with its window of 4,096 positions and prompts of 6,000 tokens).
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers N] [--dtype bf16|fp32] [--shape NAME]
                     [--prompt-len N] [--prefill-len N] [--batch B] [--points B,B] [--no-prefill]
                     [--kernels] [--ragged] [--sweep]
-    python bench.py --design situlorn|gedunex|bovozen [--sizes 2048,4096] [--kernels] [--steps K] [--warmup W]
+    python bench.py --design situlorn|gedunex|bovozen|rekirax [--sizes 2048,4096] [--kernels] [--steps K] [--warmup W]
 
 --kernels adds the time of every kernel of a decode step and of a prompt step, each taken alone at the
 shape's sizes (src/test.cpp:340-405 times single kernels so), with its rate against the peak;
@@ -20,7 +20,9 @@ Situlorn design (latent attention with and without a window, one layer on anothe
 mixture-of-experts feed-forwards) and four Llama layers of the same width and about the same weights, each a
 prompt of --prefill-len tokens and decode steps at --batch; with --kernels every kernel of both alone.  --design
 gedunex does the same for four layers of the Gedunex design (three shaped attentions under a window and one mLSTM,
-dense and mixture-of-experts feed-forwards) beside the Situlorn and the Llama layers, --design bovozen for four layers
+dense and mixture-of-experts feed-forwards) beside the Situlorn and the Llama layers, --design rekirax for four layers
+of the Rekirax design (three side-by-side mixers of a chunked rotary attention and HGRN2, one window attention, gated
+feed-forwards with biases, a way into looped layers) beside the Bovozen and the Llama layers, --design bovozen for four layers
 of the Bovozen design (two gated delta rules, two attentions inside blocks of positions, a two-matrix feed-forward and
 mixtures of experts beside a shared expert) beside the Gedunex and the Llama layers.  The default workload and its
 line stay as they are.
@@ -115,8 +117,9 @@ KERNEL_FACES = ("embed", "rmsnorm", "gemm", "gemm_norm", "gemm_norm_qkv_rope", "
                 "gemm_chain", "gemm_chain_qkv_rope", "rope_kv_write", "rope_kv_write_tiles", "attn_prefill",
                 "attn_decode", "sink_store", "attn_sink_mix", "argmax", "cast", "norm_add", "polynorm", "head_matmul",
                 "latent_pack", "moe_route", "moe_select", "moe_pair_gate_up", "moe_pair_down", "moe_grouped", "embed_sinusoid",
-                "qkv_pack", "v_tiles", "mlstm_scan", "mlstm_chunks", "gated_delta", "embed_learned", "activate", "gated_add")
-FP32_FACES = ("mlstm_scan", "mlstm_chunks", "gated_delta")     # kernels of float32 multiply-adds whatever the model's dtype: priced against that peak
+                "qkv_pack", "v_tiles", "mlstm_scan", "mlstm_chunks", "gated_delta", "embed_learned", "activate", "gated_add",
+                "time_conv", "gated_bias_act", "sigmoid_gate", "loop_pack", "hgrn2")
+FP32_FACES = ("mlstm_scan", "mlstm_chunks", "gated_delta", "hgrn2")     # kernels of float32 multiply-adds whatever the model's dtype: priced against that peak
 
 
 def record_kernel_calls(run):
@@ -226,6 +229,21 @@ def kernel_cost(name, a, kw, kv_tokens, torch):
         # per token and head: the decay, S^T k, the rank-one update and S^T q, each over the d x dv state; the operands
         # pass through memory twice (projections -> operands -> recurrence -> heads' norm), the state once each way
         return "gated_delta %d tokens" % T, nbytes(proj, low, out) + 2 * nbytes(prep, raw) + 2 * B * H * d * dv * 4, 7.0 * T * H * d * dv
+    if name == "hgrn2":
+        proj, raw, seq_slot, out = a[0], a[5], a[7], a[8]
+        H, d, dv = a[9], a[10], a[11]
+        T, B = proj.shape[0], seq_slot.shape[0]
+        # per token and head: the gate's blend and the read-out, each over the d x dv state; the read-outs pass through
+        # memory twice (recurrence -> heads' norm), the state once each way
+        return "hgrn2 %d tokens" % T, nbytes(proj, out) + 2 * nbytes(raw) + 2 * B * H * d * dv * 4, 4.0 * T * H * d * dv
+    if name == "time_conv":
+        return "time_conv %dx%d" % tuple(a[0].shape), nbytes(a[0], a[3]), 0.0
+    if name == "gated_bias_act":
+        return "gated_bias_act %dx%d" % tuple(a[0].shape), nbytes(a[0], a[2]) + (2 * nbytes(a[4]) if len(a) > 4 and a[4] is not None else 0), 0.0
+    if name == "sigmoid_gate":
+        return "sigmoid_gate %dx%d" % tuple(a[0].shape), 2 * nbytes(a[0]) + a[1].numel() * 4, 0.0
+    if name == "loop_pack":
+        return "loop_pack %dx%d" % tuple(a[0].shape), 2 * nbytes(a[0]) + nbytes(a[1], a[3]), 0.0
     if name == "activate":
         return "activate %dx%d" % tuple(a[0].shape), nbytes(a[0], a[1]), 0.0
     if name == "gated_add":
@@ -354,6 +372,25 @@ def bovozen_config(width, n_layers=4):
             "layers": [pattern[i % 4] for i in range(n_layers)]}
 
 
+def rekirax_config(width, n_layers=4):
+    """Layers of the Rekirax design at a real model's sizes: side-by-side mixers whose attention has heads of 128 in groups
+    of four, half of each head turned, inside chunks of 1,536 positions, and whose recurrence has heads of 128 x 128; a
+    window attention of the same heads over 1,024 positions; convolutions of four taps; gated feed-forwards of
+    llama_config's size; the two middle layers behind the way into a walk (walked once, so that four layers run as in
+    the designs beside it)."""
+    heads = width // 128
+    left = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": 1536},
+            "rot": {"dims": 64, "base": 500000.0}}
+    side = {"left": left, "right": {"heads": heads, "dim": 128, "vdim": 128}}
+    window = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 30.0,
+              "mask": {"size": 1024}}
+    dense = {"kind": "dense", "ff": width * 7 // 2}
+    pattern = [{"type": "parallel", "mixer": side, "mlp": dense}, {"type": "attention", "mixer": window, "mlp": dense},
+               {"type": "parallel", "mixer": side, "mlp": dense}, {"type": "parallel", "mixer": side, "mlp": dense}]
+    return {"architecture": "Rekirax", "vocab": 32000, "width": width, "norm": {"eps": 1e-5}, "canon": {"taps": 4},
+            "loop": {"start": 1, "stop": min(3, n_layers), "times": 1}, "layers": [pattern[i % 4] for i in range(n_layers)]}
+
+
 def llama_config(width, n_layers=4):
     return {"architectures": ["LlamaForCausalLM"], "hidden_size": width, "intermediate_size": width * 7 // 2,
             "num_hidden_layers": n_layers, "num_attention_heads": width // 128, "num_key_value_heads": width // 512,
@@ -372,9 +409,10 @@ def bench_design(args):
     sampler = Sampler(0)
     out = {}
     for width in [int(w) for w in args.sizes.split(",") if w]:
-        own = {"gedunex": gedunex_config, "situlorn": situlorn_config, "bovozen": bovozen_config}[args.design]
+        own = {"gedunex": gedunex_config, "situlorn": situlorn_config, "bovozen": bovozen_config, "rekirax": rekirax_config}[args.design]
         own = (args.design, own(width))
-        beside = {"gedunex": (("situlorn", situlorn_config(width)),), "bovozen": (("gedunex", gedunex_config(width)),)}.get(args.design, ())
+        beside = {"gedunex": (("situlorn", situlorn_config(width)),), "bovozen": (("gedunex", gedunex_config(width)),),
+                  "rekirax": (("bovozen", bovozen_config(width)),)}.get(args.design, ())
         for design, cfg in (own,) + beside + (("llama", llama_config(width)),):
             model = Model.random(cfg, seed=0, dtype=dtype, device="cuda:0")
             V = model.vocab_size
@@ -478,7 +516,7 @@ def main():
     ap.add_argument("--context", type=int, default=0,
                     help="the reference's -T: past this many positions two attention sinks and the last "
                          "<context> - 2 positions are attended to (0: the shape's own window, if any)")
-    ap.add_argument("--design", default="", choices=["", "situlorn", "gedunex", "bovozen"],
+    ap.add_argument("--design", default="", choices=["", "situlorn", "gedunex", "bovozen", "rekirax"],
                     help="measure layers of this design beside Llama layers of equal width instead of the default workload")
     ap.add_argument("--sizes", default="2048,4096", help="widths for --design")
     args = ap.parse_args()

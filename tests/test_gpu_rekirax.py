@@ -38,11 +38,14 @@ i32 = lambda a: torch.tensor(np.asarray(a), dtype=torch.int32, device=DEV)
 
 
 # ------------------------------------------------------------------------------------------ kernels alone
+@pytest.mark.parametrize("one_each", [False, True])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("D,taps", [(5, 1), (72, 2), (72, 4), (300, 3), (64, 16), (1030, 5)])
-def test_convolution_kernel(D, taps, dtype):
+@pytest.mark.parametrize("D,taps", [(5, 1), (72, 2), (72, 4), (300, 3), (64, 16), (1030, 5), (1024, 4)])
+def test_convolution_kernel(D, taps, dtype, one_each):
     """Two sequences and a padding row: first pieces as a step of prompts (one of them shorter than the convolution),
-    then single tokens, against the plain convolution over the whole texts; the carried inputs left behind."""
+    then single tokens, against the plain convolution over the whole texts; the carried inputs left behind.  one_each:
+    the steps of single tokens say so, and one launch then moves the carried inputs on as well (widths that are
+    multiples of eight; the others take the two launches either way)."""
     from yalm_amd.ops import kernels
     lens = [11, 7]
     hs = [randn(n, D, seed=D + i).to(dtype) for i, n in enumerate(lens)]
@@ -58,7 +61,8 @@ def test_convolution_kernel(D, taps, dtype):
         h = torch.cat(rows).to(DEV)
         out = torch.full(h.shape, float("nan"), dtype=dtype, device=DEV)
         tok_seq = [b for b in range(len(seq_slot)) for _ in range(cu[b + 1] - cu[b])]
-        kernels.time_conv(h, w.to(DEV), carried if taps > 1 else None, out, i32(tok_seq), i32(cu), i32(seq_slot))
+        kernels.time_conv(h, w.t().contiguous().to(DEV), carried if taps > 1 else None, out, i32(tok_seq), i32(cu), i32(seq_slot),
+                          one_token_each=one_each and len(tok_seq) == len(seq_slot))
         return out.float().cpu().to(F64)
 
     first = [5, 1]
@@ -82,6 +86,27 @@ def test_convolution_kernel(D, taps, dtype):
             assert torch.equal(carried[slots[b]].cpu().to(F64), held)
     if taps > 1:
         assert bool(torch.isnan(carried[1]).all()) and float(carried[3].abs().sum()) == 0.0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_convolution_kernel_over_long_prompts(dtype):
+    """Three prompts of 2,100 tokens together: the step at which a workgroup takes several tokens that follow each
+    other, across the places where one text ends and the next begins."""
+    from yalm_amd.ops import kernels
+    D, taps, lens = 64, 4, [1901, 3, 197]
+    hs = [randn(n, D, seed=i).to(dtype) for i, n in enumerate(lens)]
+    w = randn(D, taps, seed=9, scale=0.6)
+    carried = torch.zeros(3, taps - 1, D, dtype=torch.float32, device=DEV)
+    carried[1] = 1.0                              # the second text goes on from inputs of an earlier step
+    out = torch.empty(sum(lens), D, dtype=dtype, device=DEV)
+    cu = np.concatenate([[0], np.cumsum(lens)])
+    kernels.time_conv(torch.cat(hs).to(DEV), w.t().contiguous().to(DEV), carried, out, i32(np.repeat(np.arange(3), lens)), i32(cu), i32([0, 1, 2]))
+    tol = 1e-5 if dtype == torch.float32 else 3e-2
+    for b in range(3):
+        mem = {"conv": torch.ones(taps - 1, D, dtype=F64)} if b == 1 else {}
+        want = P.input_conv(hs[b].to(F64), w.to(F64), mem)
+        assert torch.allclose(out[cu[b]:cu[b + 1]].float().cpu().to(F64), want, rtol=tol, atol=tol), b
+        assert torch.equal(carried[b].cpu().to(F64), mem["conv"])
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

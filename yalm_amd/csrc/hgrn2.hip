@@ -8,9 +8,11 @@
 // hgrn2_scan: every column of S runs the recurrence on its own.  A workgroup owns 32 columns of one (sequence, head)
 // and walks the sequence's tokens of the step in order; a column is spread over eight lanes, each with NR
 // consecutive rows of it in registers (the state is kept column by column, [slot][head][column][row], so that a wave
-// reads and writes whole lines of it).  The gates of 16 tokens at a time are formed once by the whole workgroup and wait
-// in LDS, where the lanes read them four at a time; the sum over a column's rows ends with three exchanges inside
-// the eight lanes.  hgrn2_finish: the heads' norm, a wave a (token, head).
+// reads and writes whole lines of it).  The gates of 16 tokens at a time are formed once by the whole workgroup (from
+// projections that were asked for a group ahead and waited in registers) and wait in LDS, where the lanes read them
+// four at a time; a lane leaves its share of a column's read-out in LDS and goes on to the next token, and the shares
+// of a group's tokens are summed afterwards by all threads at once, so that no token waits for an exchange between
+// lanes.  hgrn2_finish: the heads' norm, a wave a (token, head).
 #include "common.h"
 #include "yalm_hip.h"
 
@@ -22,18 +24,21 @@ __global__ __launch_bounds__(SCAN_THREADS) void hgrn2_scan_kernel(
     const float* __restrict__ proj, const float* __restrict__ f_bias, const float* __restrict__ lower,
     float* __restrict__ state, float* __restrict__ raw, const int* __restrict__ cu_seqlens,
     const int* __restrict__ seq_slot, int n_heads, int d, int dv) {
-  constexpr int DP = NR * COL_LANES;              // rows as the lanes count them (zeros behind d)
+  constexpr int DP = NR * COL_LANES;              // rows as the lanes count them (zeros behind d); divides SCAN_THREADS
+  constexpr int EL = SCAN_TOKENS * DP / SCAN_THREADS;           // gates a thread forms for a group of tokens
+  constexpr int VL = SCAN_TOKENS * SCAN_COLS / SCAN_THREADS;    // values it fetches
   __shared__ float s_q[SCAN_TOKENS][DP];
   __shared__ float s_f[SCAN_TOKENS][DP];
   __shared__ float s_v[SCAN_TOKENS][SCAN_COLS];
+  __shared__ float s_part[SCAN_TOKENS][SCAN_THREADS];           // every lane's share of a column's read-out
   const int b = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * SCAN_COLS, tid = threadIdx.x;
   const int col = tid / COL_LANES, rl = tid % COL_LANES, j = c0 + col, r0 = rl * NR;
   const int slot = seq_slot[b];
   const int t0 = cu_seqlens[b], t1 = cu_seqlens[b + 1];
-  const int Hd = n_heads * d, N = 2 * Hd + n_heads * dv;
+  const int Hd = n_heads * d, HV = n_heads * dv, N = 2 * Hd + HV;
   if (slot < 0) {                                 // a padding row: no state is touched, its result is zeros
     for (int t = t0; t < t1; ++t)
-      if (rl == 0 && j < dv) raw[(size_t)t * n_heads * dv + h * dv + j] = 0.f;
+      if (rl == 0 && j < dv) raw[(size_t)t * HV + h * dv + j] = 0.f;
     return;
   }
   float* sp = state + (((size_t)slot * n_heads + h) * dv + min(j, dv - 1)) * d;      // this column's rows
@@ -49,27 +54,43 @@ __global__ __launch_bounds__(SCAN_THREADS) void hgrn2_scan_kernel(
       for (int k = 0; k < 4; ++k) s[i + k] = (r0 + i + k < d && j < dv) ? sp[r0 + i + k] : 0.f;
     }
   }
+  // the thread forms the gates of row gr of the tokens gt, gt + SCAN_THREADS / DP, ... of a group, and fetches the values
+  // of column vc of the tokens vt, vt + SCAN_THREADS / SCAN_COLS, ...: always the same row and column
+  const int gr = tid % DP, gt = tid / DP, vc = tid % SCAN_COLS, vt = tid / SCAN_COLS;
+  const bool row_ok = gr < d, col_ok = c0 + vc < dv;
+  const float fb = row_ok ? f_bias[h * d + gr] : 0.f, lo = row_ok ? lower[h * d + gr] : 0.f;
+  float zq[EL], zf[EL], zv[VL];
+  auto fetch = [&](int tc) {                      // a group's operands into registers: asked for a group ahead
+#pragma unroll
+    for (int k = 0; k < EL; ++k) {
+      const int t = tc + gt + k * (SCAN_THREADS / DP);
+      const bool ok = row_ok && t < t1;
+      zq[k] = ok ? proj[(size_t)t * N + h * d + gr] : 0.f;
+      zf[k] = ok ? proj[(size_t)t * N + Hd + h * d + gr] : 0.f;
+    }
+#pragma unroll
+    for (int k = 0; k < VL; ++k) {
+      const int t = tc + vt + k * (SCAN_THREADS / SCAN_COLS);
+      zv[k] = col_ok && t < t1 ? proj[(size_t)t * N + 2 * Hd + h * dv + c0 + vc] : 0.f;
+    }
+  };
+  fetch(t0);
   for (int tc = t0; tc < t1; tc += SCAN_TOKENS) {
     const int n = min(SCAN_TOKENS, t1 - tc);
-    __syncthreads();
-    for (int idx = tid; idx < n * DP; idx += SCAN_THREADS) {
-      const int tt = idx / DP, r = idx - tt * DP;
-      float q = 0.f, f = 0.f;
-      if (r < d) {
-        const float* row = proj + (size_t)(tc + tt) * N;
-        const float zq = row[h * d + r], zf = row[Hd + h * d + r] + f_bias[h * d + r], l = lower[h * d + r];
-        q = zq / (1.0f + expf(-zq));
-        f = l + (1.0f - l) / (1.0f + expf(-zf));
-      }
-      s_q[tt][r] = q;
-      s_f[tt][r] = f;
+    __syncthreads();                              // the group before is read
+#pragma unroll
+    for (int k = 0; k < EL; ++k) {
+      const int tt = gt + k * (SCAN_THREADS / DP);
+      const float q = zq[k] / (1.0f + expf(-zq[k]));
+      const float f = lo + (1.0f - lo) / (1.0f + expf(-(zf[k] + fb)));
+      s_q[tt][gr] = row_ok ? q : 0.f;
+      s_f[tt][gr] = row_ok ? f : 0.f;
     }
-    for (int idx = tid; idx < n * SCAN_COLS; idx += SCAN_THREADS) {
-      const int tt = idx / SCAN_COLS, c = idx - tt * SCAN_COLS;
-      s_v[tt][c] = c0 + c < dv ? proj[(size_t)(tc + tt) * N + 2 * Hd + h * dv + c0 + c] : 0.f;
-    }
+#pragma unroll
+    for (int k = 0; k < VL; ++k) s_v[vt + k * (SCAN_THREADS / SCAN_COLS)][vc] = zv[k];
+    if (tc + SCAN_TOKENS < t1) fetch(tc + SCAN_TOKENS);
     __syncthreads();
-    for (int tt = 0; tt < n; ++tt) {
+    auto token = [&](int tt) {
       const float v = s_v[tt][col];
       float acc0 = 0.f, acc1 = 0.f;
 #pragma unroll
@@ -85,11 +106,24 @@ __global__ __launch_bounds__(SCAN_THREADS) void hgrn2_scan_kernel(
         acc0 = fmaf(s[i + 2], q4.z, acc0);
         acc1 = fmaf(s[i + 3], q4.w, acc1);
       }
-      float acc = acc0 + acc1;
-      acc += __shfl_xor(acc, 1, WAVE);
-      acc += __shfl_xor(acc, 2, WAVE);
-      acc += __shfl_xor(acc, 4, WAVE);
-      if (rl == 0 && j < dv) raw[(size_t)(tc + tt) * n_heads * dv + h * dv + j] = acc;
+      s_part[tt][tid] = acc0 + acc1;
+    };
+    if (n == SCAN_TOKENS) {                       // a whole group: its tokens unrolled, so that a token's reads of LDS stand under the token before
+#pragma unroll
+      for (int tt = 0; tt < SCAN_TOKENS; ++tt) token(tt);
+    } else {
+      for (int tt = 0; tt < n; ++tt) token(tt);
+    }
+    __syncthreads();
+    // a column's read-out is the sum over its eight lanes: two (token, column) pairs a thread
+#pragma unroll
+    for (int k = 0; k < VL; ++k) {
+      const int tt = vt + k * (SCAN_THREADS / SCAN_COLS);
+      if (tt < n && col_ok) {
+        const float4 a = *reinterpret_cast<const float4*>(&s_part[tt][vc * COL_LANES]);
+        const float4 c = *reinterpret_cast<const float4*>(&s_part[tt][vc * COL_LANES + 4]);
+        raw[(size_t)(tc + tt) * HV + h * dv + c0 + vc] = ((a.x + a.y) + (a.z + a.w)) + ((c.x + c.y) + (c.z + c.w));
+      }
     }
   }
   if (j < dv) {

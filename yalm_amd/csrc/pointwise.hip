@@ -53,7 +53,8 @@ __global__ __launch_bounds__(NW * WAVE) void gated_add_kernel(const float* __res
   for (int i = threadIdx.x; i < D; i += NW * WAVE) xr[i] = accumulate ? fmaf(s, yr[i], xr[i]) : s * yr[i];
 }
 
-// out[t, c] = (residual ? h[t, c] : 0) + sum_j w[c, j] in(t - (taps - 1) + j, c): a causal convolution over the tokens
+// out[t, c] = (residual ? h[t, c] : 0) + sum_j w[j, c] in(t - (taps - 1) + j, c) (the weights tap by tap, [taps][D], so
+// that neighbouring channels' weights are neighbours): a causal convolution over the tokens
 // of a sequence, the last tap on the token itself.  Inputs in front of the step's first token of a sequence come from
 // carried[slot][taps - 1][D] (the sequence's last taps - 1 inputs, the newest last; zeros for a new sequence), and a
 // padding row (slot -1) reads zeros there.  A thread a (token, channel).
@@ -72,9 +73,85 @@ __global__ void time_conv_kernel(const T* __restrict__ h, const float* __restric
     float v = 0.f;
     if (src >= 0) v = to_f32(h[(size_t)(first + src) * D + c]);
     else if (slot >= 0) v = carried[((size_t)slot * (taps - 1) + (taps - 1 + src)) * D + c];
-    acc = fmaf(w[(size_t)c * taps + j], v, acc);
+    acc = fmaf(w[(size_t)j * D + c], v, acc);
   }
   out[(size_t)t * D + c] = from_f32<T>(acc);
+}
+
+// The same for VEC consecutive channels a thread (16 bytes of h at a time), D a multiple of VEC.  one_each: every
+// sequence brings one token (row t is sequence t), and the thread also moves the carried inputs on: it has read the
+// old ones before it writes, and nobody else touches its channels.
+template <typename T, int VEC> struct Chunk;
+template <> struct Chunk<float, 4> {
+  static __device__ __forceinline__ void load(const float* p, float* v) {
+    const float4 x = *reinterpret_cast<const float4*>(p);
+    v[0] = x.x, v[1] = x.y, v[2] = x.z, v[3] = x.w;
+  }
+  static __device__ __forceinline__ void store(float* p, const float* v) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  }
+};
+template <> struct Chunk<bf16, 8> {
+  typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+  static __device__ __forceinline__ void load(const bf16* p, float* v) {
+    const bf16x8 x = *reinterpret_cast<const bf16x8*>(p);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] = static_cast<float>(x[k]);
+  }
+  static __device__ __forceinline__ void store(bf16* p, const float* v) {
+    bf16x8 x;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) x[k] = static_cast<bf16>(v[k]);
+    *reinterpret_cast<bf16x8*>(p) = x;
+  }
+};
+template <typename E, int VEC>
+__global__ void time_conv_vec_kernel(const E* __restrict__ h, const float* __restrict__ w, float* __restrict__ carried,
+                                     E* __restrict__ out, const int* __restrict__ tok_seq,
+                                     const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slot, int D, int taps,
+                                     int residual, int one_each, int n_tokens, int per_block) {
+  const int c = (blockIdx.y * blockDim.x + threadIdx.x) * VEC;
+  if (c >= D) return;
+  // a workgroup takes per_block tokens that follow each other: a token's earlier inputs are then lines that the
+  // same threads have just read
+  for (int t = blockIdx.x * per_block; t < min(n_tokens, (int)(blockIdx.x + 1) * per_block); ++t) {
+  const int b = one_each ? t : tok_seq[t];
+  const int first = one_each ? t : (b >= 0 ? cu_seqlens[b] : t), slot = b >= 0 ? seq_slot[b] : -1;
+  const int l = t - first, keep = taps - 1;
+  float own[VEC], acc[VEC], v[VEC];
+  Chunk<E, VEC>::load(h + (size_t)t * D + c, own);
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) acc[k] = residual ? own[k] : 0.f;
+  for (int j = 0; j < taps; ++j) {
+    const int src = l - keep + j;
+    if (src >= 0) {
+      Chunk<E, VEC>::load(h + (size_t)(first + src) * D + c, v);
+    } else if (slot >= 0) {
+      const float* row = carried + ((size_t)slot * keep + (keep + src)) * D + c;
+#pragma unroll
+      for (int k = 0; k < VEC; k += 4) Chunk<float, 4>::load(row + k, v + k);
+      if (one_each && j > 0) {                    // the row moves one place towards the oldest
+        float* older = carried + ((size_t)slot * keep + (keep + src - 1)) * D + c;
+#pragma unroll
+        for (int k = 0; k < VEC; k += 4) Chunk<float, 4>::store(older + k, v + k);
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) v[k] = 0.f;
+    }
+    float wj[VEC];
+#pragma unroll
+    for (int k = 0; k < VEC; k += 4) Chunk<float, 4>::load(w + (size_t)j * D + c + k, wj + k);
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) acc[k] = fmaf(wj[k], v[k], acc[k]);
+  }
+  if (one_each && slot >= 0 && keep > 0) {        // the token itself is the newest carried input
+    float* newest = carried + ((size_t)slot * keep + (keep - 1)) * D + c;
+#pragma unroll
+    for (int k = 0; k < VEC; k += 4) Chunk<float, 4>::store(newest + k, own + k);
+  }
+  Chunk<E, VEC>::store(out + (size_t)t * D + c, acc);
+  }
 }
 
 // carried[slot] <- the last taps - 1 inputs of each sequence after this step's tokens; a thread a (sequence, channel)
@@ -104,13 +181,13 @@ __global__ void time_conv_carry_kernel(const T* __restrict__ h, float* __restric
 
 // out[t, i] = act(z[t, i] + bias[i]) * (z[t, F + i] + bias[F + i]) for i < F: the middle of a gated feed-forward whose
 // two first products (gate | up, float32) carry biases; x[t, :] += x_bias (the second product's bias, which that
-// product's adding epilogue does not know) on the way.  A workgroup a token.
+// product's adding epilogue does not know) on the way.  A workgroup a token, or several where the tokens are few.
 template <typename T>
 __global__ void gated_bias_act_kernel(const float* __restrict__ z, const float* __restrict__ bias, T* __restrict__ out,
                                       int F, int kind, float* __restrict__ x, const float* __restrict__ x_bias, int D) {
-  const int t = blockIdx.x;
+  const int t = blockIdx.x, first = blockIdx.y * blockDim.x + threadIdx.x, stride = gridDim.y * blockDim.x;
   const float* zr = z + (size_t)t * 2 * F;
-  for (int i = threadIdx.x; i < F; i += blockDim.x) {
+  for (int i = first; i < F; i += stride) {
     const float v = zr[i] + (bias != nullptr ? bias[i] : 0.f), u = zr[F + i] + (bias != nullptr ? bias[F + i] : 0.f);
     float a;
     if (kind == 0) a = 0.5f * v * (1.0f + erff(v * 0.7071067811865476f));
@@ -119,7 +196,7 @@ __global__ void gated_bias_act_kernel(const float* __restrict__ z, const float* 
     out[(size_t)t * F + i] = from_f32<T>(a * u);
   }
   if (x_bias != nullptr)
-    for (int i = threadIdx.x; i < D; i += blockDim.x) x[(size_t)t * D + i] += x_bias[i];
+    for (int i = first; i < D; i += stride) x[(size_t)t * D + i] += x_bias[i];
 }
 
 // o[t, h, e] *= sigmoid(g[t * g_stride + h * dv + e]) for e < dv (heads of o are `pad` wide); a workgroup a token
@@ -200,11 +277,30 @@ extern "C" int yalm_gated_add(const float* y, const void* h, const void* w, int 
 constexpr int CONV_MAX_TAPS = 16;
 extern "C" int yalm_time_conv(const void* h, const float* w, float* carried, void* out, const int* tok_seq,
                               const int* cu_seqlens, const int* seq_slot, int T, int B, int D, int taps, int residual,
-                              int dtype, hipStream_t stream) {
+                              int one_each, int dtype, hipStream_t stream) {
   if (T <= 0) return YALM_OK;
+  if (one_each && T != B) return YALM_ERR_ARG;
   if (D <= 0 || B <= 0 || taps <= 0 || taps > CONV_MAX_TAPS || h == out ||
       (taps > 1 && carried == nullptr) || ceil_div(D, 256) > 65535)
     return YALM_ERR_ARG;
+  const int vec = dtype == YALM_F32 ? 4 : 8;
+  if (D % vec == 0 && (((uintptr_t)h | (uintptr_t)out | (uintptr_t)carried) & 15) == 0 && (dtype == YALM_F32 || dtype == YALM_BF16)) {
+    const int lanes = D / vec, vthreads = lanes >= 256 ? 256 : 64;
+    const int per_block = (long)T * D >= 2048L * 4096 ? 4 : 1;      // measured: 20.1 -> 15.8 us at 2,048 x 4,096, no gain below
+    dim3 vgrid(ceil_div(T, per_block), ceil_div(lanes, vthreads)), vcgrid(B, ceil_div(D, 256));
+    if (dtype == YALM_F32) {
+      time_conv_vec_kernel<float, 4><<<vgrid, vthreads, 0, stream>>>((const float*)h, w, carried, (float*)out, tok_seq, cu_seqlens,
+                                                                    seq_slot, D, taps, residual, one_each, T, per_block);
+      if (taps > 1 && !one_each)
+        time_conv_carry_kernel<float, CONV_MAX_TAPS><<<vcgrid, 256, 0, stream>>>((const float*)h, carried, cu_seqlens, seq_slot, D, taps);
+    } else {
+      time_conv_vec_kernel<bf16, 8><<<vgrid, vthreads, 0, stream>>>((const bf16*)h, w, carried, (bf16*)out, tok_seq, cu_seqlens,
+                                                                   seq_slot, D, taps, residual, one_each, T, per_block);
+      if (taps > 1 && !one_each)
+        time_conv_carry_kernel<bf16, CONV_MAX_TAPS><<<vcgrid, 256, 0, stream>>>((const bf16*)h, carried, cu_seqlens, seq_slot, D, taps);
+    }
+    return launch_status();
+  }
   const int threads = D >= 256 ? 256 : 64;
   dim3 grid(T, ceil_div(D, threads)), cgrid(B, ceil_div(D, threads));
   if (dtype == YALM_F32) {
@@ -227,11 +323,14 @@ extern "C" int yalm_gated_bias_act(const float* z, const float* bias, void* out,
                                    float* x, const float* x_bias, int D, hipStream_t stream) {
   if (T <= 0) return YALM_OK;
   if (F <= 0 || kind < 0 || kind > 2 || (x_bias != nullptr && (x == nullptr || D <= 0))) return YALM_ERR_ARG;
-  const int threads = F >= 2048 ? 1024 : 256;
+  const int threads = 256;
+  int slices = T >= 512 ? 1 : ceil_div(512, T);                   // a step of few tokens still fills the chip
+  slices = slices < ceil_div(F, threads) ? slices : ceil_div(F, threads);
+  dim3 grid(T, slices > 0 ? slices : 1);
   if (out_dtype == YALM_F32)
-    gated_bias_act_kernel<float><<<T, threads, 0, stream>>>(z, bias, (float*)out, F, kind, x, x_bias, D);
+    gated_bias_act_kernel<float><<<grid, threads, 0, stream>>>(z, bias, (float*)out, F, kind, x, x_bias, D);
   else if (out_dtype == YALM_BF16)
-    gated_bias_act_kernel<bf16><<<T, threads, 0, stream>>>(z, bias, (bf16*)out, F, kind, x, x_bias, D);
+    gated_bias_act_kernel<bf16><<<grid, threads, 0, stream>>>(z, bias, (bf16*)out, F, kind, x, x_bias, D);
   else
     return YALM_ERR_DTYPE;
   return launch_status();

@@ -147,7 +147,8 @@ template <> struct Pack4<bf16> {
 };
 constexpr int PW_WAVES = 4;
 
-template <typename T, int NV>
+// SHAPED: with norms a head, values that are the keys, or the rotation (the other models run the code without them)
+template <typename T, int NV, bool SHAPED>
 __global__ __launch_bounds__(PW_WAVES * WAVE) void qkv_pack_wave_kernel(
     const float* __restrict__ qkv, const float* __restrict__ bias, const float* __restrict__ w_q,
     const float* __restrict__ w_k, float eps, float temp_coef, int temp_every, float q_scale, float* __restrict__ v_first,
@@ -155,10 +156,13 @@ __global__ __launch_bounds__(PW_WAVES * WAVE) void qkv_pack_wave_kernel(
     const int* __restrict__ seq_tile0, T* __restrict__ k_pages, T* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, int ring_pages, const int* __restrict__ tok_seq,
     const int* __restrict__ tok_pos, const int* __restrict__ seq_slot, const int* __restrict__ seq_len, int n_tokens,
-    int n_heads, int n_kv_heads, int d, int dv, int pad, int n_pages, int page_layout, T* __restrict__ v_rows) {
+    int n_heads, int n_kv_heads, int d, int dv, int pad, int n_pages, int page_layout, T* __restrict__ v_rows,
+    int head_norm_, int v_from_k_, const float2* __restrict__ cos_sin, int rot_dims_, int n_positions) {
+  // head_norm here: d a power of two from 4 to 256, so that a head's elements lie in d / 4 neighbouring lanes of one round
+  const int head_norm = SHAPED ? head_norm_ : 0, v_from_k = SHAPED ? v_from_k_ : 0, rot_dims = SHAPED ? rot_dims_ : 0;
   const int t = blockIdx.x * PW_WAVES + threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   if (t >= n_tokens) return;
-  const int Q = n_heads * d, K = n_kv_heads * d, V = n_kv_heads * dv, N = Q + K + V;
+  const int Q = n_heads * d, K = n_kv_heads * d, V = n_kv_heads * dv, N = Q + K + (v_from_k ? 0 : V);
   const float* src = qkv + (size_t)t * N;
   float4 r[NV], wt[NV];                           // the row and the norm weights of its elements: every load asked for at once
   float sq = 0.f, sk = 0.f;
@@ -166,9 +170,10 @@ __global__ __launch_bounds__(PW_WAVES * WAVE) void qkv_pack_wave_kernel(
   for (int j = 0; j < NV; ++j) {
     const int i = (j * WAVE + lane) * 4;
     wt[j] = make_float4(1.f, 1.f, 1.f, 1.f);
-    if (i < Q && w_q != nullptr) wt[j] = *reinterpret_cast<const float4*>(w_q + i);
-    else if (i >= Q && i < Q + K && w_k != nullptr) wt[j] = *reinterpret_cast<const float4*>(w_k + (i - Q));
+    if (i < Q && w_q != nullptr) wt[j] = *reinterpret_cast<const float4*>(w_q + (head_norm ? i % d : i));
+    else if (i >= Q && i < Q + K && w_k != nullptr) wt[j] = *reinterpret_cast<const float4*>(w_k + (head_norm ? (i - Q) % d : i - Q));
   }
+
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
     const int i = (j * WAVE + lane) * 4;
@@ -184,6 +189,14 @@ __global__ __launch_bounds__(PW_WAVES * WAVE) void qkv_pack_wave_kernel(
       else if (i < Q + K) sk += ss;
     }
     r[j] = v;
+    if constexpr (SHAPED) {
+      if (head_norm) {                            // the sum over the head's lanes (neighbours: exchanges inside their group);
+        float ss = i < Q + K ? v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w : 0.f;      // 1 / rms rides on the norm's weights
+        for (int o = 1; o < d / 4; o <<= 1) ss += __shfl_xor(ss, o, WAVE);
+        const float f = 1.0f / sqrtf(ss / (float)d + eps);
+        wt[j].x *= f, wt[j].y *= f, wt[j].z *= f, wt[j].w *= f;
+      }
+    }
   }
   sq = wave_sum(sq);
   sk = wave_sum(sk);
@@ -191,11 +204,25 @@ __global__ __launch_bounds__(PW_WAVES * WAVE) void qkv_pack_wave_kernel(
   const int b = tok_seq[t];
   const int slot = b >= 0 ? seq_slot[b] : -1;
   float fq = q_scale;
-  if (w_q != nullptr) fq *= 1.0f / sqrtf(sq / (float)Q + eps);
+  if (w_q != nullptr && !head_norm) fq *= 1.0f / sqrtf(sq / (float)Q + eps);
   if (temp_every > 0) fq *= 1.0f + temp_coef * logf((float)((pos + 1) / temp_every) + 1.0f);
-  const float fk = w_k != nullptr ? 1.0f / sqrtf(sk / (float)K + eps) : 1.0f;
+  const float fk = w_k != nullptr && !head_norm ? 1.0f / sqrtf(sk / (float)K + eps) : 1.0f;
   const float lam = blend == 2 ? lam_p[0] : 0.f;
   const int row = pos & (PAGE - 1);
+  const float2* cs = rot_dims > 0 ? cos_sin + (size_t)min(max(pos, 0), n_positions - 1) * (rot_dims / 2) : nullptr;
+  // the lane's four elements e .. e + 3 of a head are two of the rotation's pairs
+  auto turn = [&](int e, float& a0, float& a1, float& a2, float& a3) {
+    if (e < rot_dims) {
+      const float2 c = cs[e >> 1];
+      const float x = a0 * c.x - a1 * c.y, y = a1 * c.x + a0 * c.y;
+      a0 = x, a1 = y;
+    }
+    if (e + 2 < rot_dims) {
+      const float2 c = cs[(e >> 1) + 1];
+      const float x = a2 * c.x - a3 * c.y, y = a3 * c.x + a2 * c.y;
+      a2 = x, a3 = y;
+    }
+  };
   long page = -1, tile = -1;
   if (slot >= 0 && pos >= 0 && k_pages != nullptr) {
     const int ap = pos / PAGE, last_ap = (seq_len[b] - 1) / PAGE;
@@ -214,11 +241,27 @@ __global__ __launch_bounds__(PW_WAVES * WAVE) void qkv_pack_wave_kernel(
     if (i < Q) {
       const int h = i / d, e = i - h * d;
       const float4 w4 = wt[j];
-      Pack4<T>::store(qo + h * pad + e, v.x * fq * w4.x, v.y * fq * w4.y, v.z * fq * w4.z, v.w * fq * w4.w);
+      float a0 = v.x * fq * w4.x, a1 = v.y * fq * w4.y, a2 = v.z * fq * w4.z, a3 = v.w * fq * w4.w;
+      if constexpr (SHAPED) turn(e, a0, a1, a2, a3);
+      Pack4<T>::store(qo + h * pad + e, a0, a1, a2, a3);
     } else if (i < Q + K) {
       const int ik = i - Q, g = ik / d, e = ik - g * d;
       const float4 w4 = wt[j];
-      const float a0 = v.x * fk * w4.x, a1 = v.y * fk * w4.y, a2 = v.z * fk * w4.z, a3 = v.w * fk * w4.w;
+      float a0 = v.x * fk * w4.x, a1 = v.y * fk * w4.y, a2 = v.z * fk * w4.z, a3 = v.w * fk * w4.w;
+      if constexpr (SHAPED) turn(e, a0, a1, a2, a3);
+      if (SHAPED && v_from_k) {                             // the key as projected is the value
+        if (v_rows != nullptr) {
+          Pack4<T>::store(v_rows + (size_t)t * n_kv_heads * pad + g * pad + e, v.x, v.y, v.z, v.w);
+        } else {
+          const float vals[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const T vt = from_f32<T>(vals[u]);
+            if (tile >= 0) v_stage[((size_t)tile * n_kv_heads + g) * PAGE * pad + (size_t)(e + u) * PAGE + row] = vt;
+            if (page >= 0) v_pages[((size_t)page * n_kv_heads + g) * PAGE * pad + page_v_offset(page_layout, row, e + u, pad)] = vt;
+          }
+        }
+      }
       if (tile >= 0) Pack4<T>::store(k_stage + ((size_t)tile * n_kv_heads + g) * PAGE * pad + (size_t)row * pad + e, a0, a1, a2, a3);
       if (page >= 0)                              // four consecutive elements lie together in either layout
         Pack4<T>::store(k_pages + ((size_t)page * n_kv_heads + g) * PAGE * pad + page_k_offset(page_layout, row, e, pad), a0, a1, a2, a3);
@@ -374,16 +417,21 @@ extern "C" int yalm_qkv_pack(const float* qkv, const float* bias, const float* w
   if (lds > 64 * 1024) return YALM_ERR_ARG;
   // a wave a token where a lane can take four elements at a time and the row fits its registers, and where the tokens
   // are many: a few tokens are done sooner by 1,024 threads each (8 tokens of 6,144 numbers: 12 against 25 us)
-  const bool by_wave = !head_norm && !v_from_k && rot_dims == 0 && T >= 32 && d % 4 == 0 && dv % 4 == 0 && n_row <= 256 * 32 &&
+  const bool heads_fit = !head_norm || (d >= 4 && d <= 256 && (d & (d - 1)) == 0);      // a head in neighbouring lanes
+  const bool by_wave = heads_fit && T >= 32 && d % 4 == 0 && dv % 4 == 0 && n_row <= 256 * 32 &&
                        ((((uintptr_t)qkv) | ((uintptr_t)bias) | ((uintptr_t)w_q) | ((uintptr_t)w_k) | ((uintptr_t)v_first) |
                          ((uintptr_t)q_out) | ((uintptr_t)k_stage) | ((uintptr_t)k_pages) | ((uintptr_t)v_rows)) & 15) == 0;
   if (by_wave) {
     const int blocks = ceil_div(T, PW_WAVES);
+    const bool shaped = head_norm || v_from_k || rot_dims > 0;
 #define YALM_PACK_W(TYPE, NV_)                                                                                           \
-  qkv_pack_wave_kernel<TYPE, NV_><<<blocks, PW_WAVES * WAVE, 0, stream>>>(                                               \
+  do { if (shaped) YALM_PACK_WS(TYPE, NV_, true); else YALM_PACK_WS(TYPE, NV_, false); } while (0)
+#define YALM_PACK_WS(TYPE, NV_, SHAPED_)                                                                                 \
+  qkv_pack_wave_kernel<TYPE, NV_, SHAPED_><<<blocks, PW_WAVES * WAVE, 0, stream>>>(                                               \
       qkv, bias, w_q, w_k, eps, temp_coef, temp_every, q_scale, v_first, blend, lam, (TYPE*)q_out, (TYPE*)k_stage,        \
       (TYPE*)v_stage, seq_tile0, (TYPE*)k_pages, (TYPE*)v_pages, block_table, table_stride, ring_pages, tok_seq,         \
-      tok_pos, seq_slot, seq_len, T, n_heads, n_kv_heads, d, dv, pad, n_pages, page_layout, (TYPE*)v_rows)
+      tok_pos, seq_slot, seq_len, T, n_heads, n_kv_heads, d, dv, pad, n_pages, page_layout, (TYPE*)v_rows, head_norm,    \
+      v_from_k, (const float2*)cos_sin, rot_dims, n_positions)
 #define YALM_PACK_WN(TYPE)                                                                                               \
   if (n_row <= 256 * 4) YALM_PACK_W(TYPE, 4);                                                                            \
   else if (n_row <= 256 * 8) YALM_PACK_W(TYPE, 8);                                                                       \
@@ -399,6 +447,7 @@ extern "C" int yalm_qkv_pack(const float* qkv, const float* bias, const float* w
     }
 #undef YALM_PACK_WN
 #undef YALM_PACK_W
+#undef YALM_PACK_WS
     return launch_status();
   }
   const bool wide = n_row >= 2048;

@@ -385,12 +385,13 @@ int yalm_activate(const float* z, void* out, long n, int kind, int out_dtype, hi
 // x[t, :] (+)= sigmoid(h[t, :] . w) * y[t, :]; h [T, D] and w [D] of `dtype`, x and y float32; accumulate 0: x is written.
 int yalm_gated_add(const float* y, const void* h, const void* w, int dtype, float* x, int T, int D, int accumulate,
                    hipStream_t stream);
-// out[t, c] = (residual ? h[t, c] : 0) + sum_j w[c, j] in(t - (taps - 1) + j, c): a causal convolution over the tokens of
-// each sequence (h, out [T, D] of `dtype`, not the same memory; w float32 [D, taps], the last tap on the token itself).
+// out[t, c] = (residual ? h[t, c] : 0) + sum_j w[j, c] in(t - (taps - 1) + j, c): a causal convolution over the tokens of
+// each sequence (h, out [T, D] of `dtype`, not the same memory; w float32 [taps, D], tap by tap, the last tap on the token itself).
 // carried, float32 [n_slots, taps - 1, D], holds each sequence's last taps - 1 inputs (the newest last): read for the
 // places in front of the step's first token, then left advanced.  Rows of padding (slot -1) read zeros and keep nothing.
+// one_each != 0: every sequence brings one token (T = B, row t is sequence t), which lets one launch do both.
 int yalm_time_conv(const void* h, const float* w, float* carried, void* out, const int* tok_seq, const int* cu_seqlens,
-                   const int* seq_slot, int T, int B, int D, int taps, int residual, int dtype, hipStream_t stream);
+                   const int* seq_slot, int T, int B, int D, int taps, int residual, int one_each, int dtype, hipStream_t stream);
 // out[t, i] = act(z[t, i] + bias[i]) * (z[t, F + i] + bias[F + i]), i < F: z float32 [T, 2 F] (gate | up), bias float32
 // [2 F] or null, out of `out_dtype`, kind as yalm_activate; with x_bias (float32 [D]) also x[t, :] += x_bias (x float32 [T, D]).
 int yalm_gated_bias_act(const float* z, const float* bias, void* out, int T, int F, int kind, int out_dtype, float* x,

@@ -1089,13 +1089,14 @@ def gated_add(y, h, w, x, accumulate=True):
 TIME_CONV_MAX_TAPS = 16
 
 
-def time_conv(h, w, carried, out, tok_seq, cu_seqlens, seq_slot, residual=True):
-    """out[t, c] = (h[t, c] if residual) + sum_j w[c, j] in(t - (taps - 1) + j, c): a causal convolution over the tokens
+def time_conv(h, w, carried, out, tok_seq, cu_seqlens, seq_slot, residual=True, one_token_each=False):
+    """out[t, c] = (h[t, c] if residual) + sum_j w[j, c] in(t - (taps - 1) + j, c): a causal convolution over the tokens
     of each sequence of the step, the last tap on the token itself (h, out [T, D] of one dtype and not the same
-    memory; w float32 [D, taps]).  carried (float32 [slots, taps - 1, D]; None with one tap) holds each sequence's last
-    taps - 1 inputs, read for the places in front of the step's first token and left advanced."""
+    memory; w float32 [taps, D], tap by tap).  carried (float32 [slots, taps - 1, D]; None with one tap) holds each sequence's last
+    taps - 1 inputs, read for the places in front of the step's first token and left advanced.  one_token_each: the caller
+    knows that every sequence brings one token (row t is sequence t), which saves a launch."""
     T, D = h.shape
-    taps = w.shape[1]
+    taps = w.shape[0]
     B = seq_slot.shape[0]
     if not 0 < taps <= TIME_CONV_MAX_TAPS:
         raise ValueError("time_conv: %d taps (at most %d)" % (taps, TIME_CONV_MAX_TAPS))
@@ -1105,9 +1106,10 @@ def time_conv(h, w, carried, out, tok_seq, cu_seqlens, seq_slot, residual=True):
     if taps > 1:
         p_c = _need(carried, "carried", torch.float32, (None, taps - 1, D))
     library.check(library.lib().yalm_time_conv(
-        _need(h, "h", None, (T, D)), _need(w, "w", torch.float32, (D, taps)), p_c, _need(out, "out", h.dtype, (T, D)),
+        _need(h, "h", None, (T, D)), _need(w, "w", torch.float32, (taps, D)), p_c, _need(out, "out", h.dtype, (T, D)),
         _need(tok_seq, "tok_seq", torch.int32, (T,)), _need(cu_seqlens, "cu_seqlens", torch.int32, (B + 1,)),
-        _need(seq_slot, "seq_slot", torch.int32, (B,)), T, B, D, taps, 1 if residual else 0, dtype_code(h.dtype), _stream()),
+        _need(seq_slot, "seq_slot", torch.int32, (B,)), T, B, D, taps, 1 if residual else 0,
+        1 if one_token_each and T == B else 0, dtype_code(h.dtype), _stream()),
         "time_conv")
     return out
 

@@ -73,7 +73,7 @@ _SIGNATURES = {
     "yalm_embed_learned": (_I, [_P, _P, _I, _P, _P, _F, _P, _I, _I, _I, _I, _P]),
     "yalm_activate": (_I, [_P, _P, ctypes.c_long, _I, _I, _P]),
     "yalm_gated_add": (_I, [_P, _P, _P, _I, _P, _I, _I, _I, _P]),
-    "yalm_time_conv": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]),
+    "yalm_time_conv": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_gated_bias_act": (_I, [_P, _P, _P, _I, _I, _I, _I, _P, _P, _I, _P]),
     "yalm_sigmoid_gate": (_I, [_P, _P, ctypes.c_long, _I, _I, _I, _I, _I, _P]),
     "yalm_loop_pack": (_I, [_P, _P, _P, _P, _I, _I, _I, _P]),
@@ -82,7 +82,7 @@ _SIGNATURES = {
     "yalm_probe_mfma": (_I, [_I, _I, _I, _P, _P, _P]),
 }
 
-ABI_VERSION = 34
+ABI_VERSION = 35
 
 
 class KernelError(RuntimeError):

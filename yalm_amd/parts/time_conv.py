@@ -25,7 +25,7 @@ class TimeConv(Part):
         return [ParamSpec(self.tensor, (self.dim, self.taps), init="taps")]
 
     def load(self, get, compute_dtype, device):
-        self.w = get(self.tensor).to(torch.float32).to(device).contiguous()
+        self.w = get(self.tensor).to(torch.float32).t().contiguous().to(device)      # tap by tap: [taps, dim]
 
     def weight_bytes(self):
         return self.dim * self.taps * 4
@@ -36,4 +36,5 @@ class TimeConv(Part):
     def forward(self, h, out, ctx, line):
         """out = h (+) conv(h) over the step's tokens, from the inputs that the line's state holds, which it leaves advanced."""
         carried = ctx.cache.group_of(line).line_state(line) if self.taps > 1 else None
-        return kernels.time_conv(h, self.w, carried, out, ctx.tok_seq, ctx.cu_seqlens, ctx.seq_slot, self.residual)
+        return kernels.time_conv(h, self.w, carried, out, ctx.tok_seq, ctx.cu_seqlens, ctx.seq_slot, self.residual,
+                                 one_token_each=ctx.mode == "decode")
