@@ -76,6 +76,15 @@ PLAIN = model(80, 32, 1e-5, [                     # no convolution, no loop
     layer(par(2, 2, 16, 16, 0.25, chunk=16, rot=8, right=(2, 8, 16)), dense(48)),
 ])
 
+# heads of the sizes the matrix-core attention and the wave-a-token packing kernel are built for, a chunk and a window that
+# cross pages, recurrent heads of 32 channels
+MEDIUM = model(500, 256, 1e-5, [
+    layer(par(4, 2, 64, 64, 0.125, chunk=100, rot=32, base=500000.0, right=(4, 32, 64)), dense(512)),
+    layer(win(4, 1, 128, 0.09, window=200, softcap=20.0), dense(384)),
+    layer(par(8, 8, 32, 32, 0.18, chunk=64, rot=32, right=(2, 64, 32)), dense(512)),
+    layer(par(4, 2, 64, 64, 0.125, chunk=130, rot=16, right=(4, 32, 64)), None),
+], taps=4, loop=(1, 3, 2))
+
 # one mechanism at a time
 ONLY_WINDOW = model(90, 40, 1e-5, [layer(win(2, 1, 16, 0.4, window=7, softcap=20.0), dense(32))], taps=1)
 ONLY_WIDE_WINDOW = model(90, 40, 1e-5, [layer(win(2, 2, 32, 0.3, window=150, softcap=20.0), None)], taps=1)
@@ -88,6 +97,6 @@ ONLY_CONV = model(90, 40, 1e-5, [layer(win(2, 1, 8, 0.4, window=1), dense(32))],
 ONLY_FULL = model(90, 48, 1e-5, [layer(win(2, 1, 64, 0.2, softcap=40.0), dense(32))], taps=2)
 LOOPED = model(90, 40, 1e-5, [layer(par(2, 1, 8, 8, 0.4, chunk=12, rot=8, right=(2, 8, 8)), dense(32))], taps=2, loop=(0, 1, 3))
 
-ALL = {"mixed": MIXED, "windows": WINDOWS, "chunks": CHUNKS, "odd": ODD, "plain": PLAIN, "only_window": ONLY_WINDOW,
+ALL = {"mixed": MIXED, "medium": MEDIUM, "windows": WINDOWS, "chunks": CHUNKS, "odd": ODD, "plain": PLAIN, "only_window": ONLY_WINDOW,
        "only_wide_window": ONLY_WIDE_WINDOW, "only_chunk": ONLY_CHUNK, "only_wide_chunk": ONLY_WIDE_CHUNK,
        "only_state": ONLY_STATE, "only_conv": ONLY_CONV, "only_full": ONLY_FULL, "looped": LOOPED}

@@ -421,11 +421,12 @@ def compare(folders, name, dtype, steps, requests, engine, what):
         assert g.pool.n_free == g.n_pages
 
 
-LENGTHS = {"mixed": [1, 2, 23, 64, 65, 150, 230], "windows": [1, 5, 6, 64, 66, 131, 200], "chunks": [1, 7, 8, 65, 129, 180],
+LENGTHS = {"mixed": [1, 2, 23, 64, 65, 150, 230], "medium": [300, 70, 131], "windows": [1, 5, 6, 64, 66, 131, 200], "chunks": [1, 7, 8, 65, 129, 180],
            "odd": [1, 9, 10, 70, 129], "plain": [1, 17, 40], "only_window": [3, 7, 8, 70], "only_wide_window": [149, 151, 301],
            "only_chunk": [3, 7, 8, 70], "only_wide_chunk": [149, 151, 301], "only_state": [1, 2, 70], "only_conv": [1, 3, 4, 30],
            "only_full": [2, 130], "looped": [1, 13, 40]}
 GROUPS = {"mixed": [([0, 2, 4, 5], [1, 23, 60, 100]), ([6, 1, 3], [221, 2, 64]), ([5, 4], [2, 1])],
+          "medium": [([0, 1, 2], [250, 3, 100]), ([2, 1], [1, 64])],
           "windows": [([0, 1, 2, 3], [1, 5, 2, 64]), ([4, 5, 6], [63, 100, 130]), ([6, 5], [190, 1])],
           "chunks": [([0, 1, 2, 3], [1, 7, 3, 64]), ([4, 5], [100, 130]), ([5, 3], [170, 1])],
           "odd": [([0, 1, 2, 3], [1, 3, 10, 64]), ([4, 3], [100, 1])],
