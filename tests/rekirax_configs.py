@@ -79,10 +79,10 @@ PLAIN = model(80, 32, 1e-5, [                     # no convolution, no loop
 # heads of the sizes the matrix-core attention and the wave-a-token packing kernel are built for, a chunk and a window that
 # cross pages, recurrent heads of 32 channels
 MEDIUM = model(500, 256, 1e-5, [
-    layer(par(4, 2, 64, 64, 0.125, chunk=100, rot=32, base=500000.0, right=(4, 32, 64)), dense(512)),
+    layer(par(4, 2, 64, 64, 0.11, chunk=100, rot=32, base=250000.0, right=(4, 32, 48)), dense(512)),
     layer(win(4, 1, 128, 0.09, window=200, softcap=20.0), dense(384)),
     layer(par(8, 8, 32, 32, 0.18, chunk=64, rot=32, right=(2, 64, 32)), dense(512)),
-    layer(par(4, 2, 64, 64, 0.125, chunk=130, rot=16, right=(4, 32, 64)), None),
+    layer(par(4, 2, 64, 64, 0.14, chunk=130, rot=24, right=(3, 32, 80)), None),
 ], taps=4, loop=(1, 3, 2))
 
 # one mechanism at a time
